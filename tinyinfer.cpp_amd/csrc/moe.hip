@@ -15,6 +15,7 @@ TI_ERROR_API
 // score kinds
 #define MOE_SIGMOID 0
 #define MOE_SOFTMAX 1
+#define MOE_SOFTMAX_CHOSEN 2      // the largest logits are chosen; the weights are the softmax over the chosen logits alone
 
 template <typename T> struct Piece;
 template <> struct Piece<float> {
@@ -81,12 +82,12 @@ moe_route_kernel(const T* __restrict__ h, const float* __restrict__ router, int*
     for (int e = threadIdx.x; e < E; e += 256) sum += expf(s_score[e] - mx);
     sum = block_sum<256>(sum, red);
     for (int e = threadIdx.x; e < E; e += 256) s_score[e] = expf(s_score[e] - mx) / sum;
-  } else {
+  } else if (score_kind == MOE_SIGMOID) {
     for (int e = threadIdx.x; e < E; e += 256) s_score[e] = 1.0f / (1.0f + expf(-s_score[e]));
   }
   __syncthreads();
   if (wave != 0) return;
-  float total = 0.f;
+  float total = 0.f, first = 0.f;
   for (int k = 0; k < top; ++k) {
     float best = -INFINITY;
     int at = 0x7fffffff;
@@ -111,11 +112,19 @@ moe_route_kernel(const T* __restrict__ h, const float* __restrict__ router, int*
       wts[(size_t)m * top + k] = best;
       s_score[at] = -INFINITY;
     }
-    total += best;
+    if (score_kind == MOE_SOFTMAX_CHOSEN) {
+      // the first choice is the largest logit: every weight is exp(z - z_first) over the sum of those, in the order of choice
+      if (k == 0) first = best;
+      const float w = expf(best - first);
+      if (lane == 0) wts[(size_t)m * top + k] = w;
+      total += w;
+    } else {
+      total += best;
+    }
     __builtin_amdgcn_wave_barrier();
     __threadfence_block();
   }
-  if (renormalize && lane < top) wts[(size_t)m * top + lane] /= total;
+  if ((renormalize || score_kind == MOE_SOFTMAX_CHOSEN) && lane < top) wts[(size_t)m * top + lane] /= total;
 }
 
 extern "C" int ti_moe_route(int dtype, const void* h, const float* router, int* ids, float* wts, int M, int W, int E, int top,
@@ -123,7 +132,7 @@ extern "C" int ti_moe_route(int dtype, const void* h, const float* router, int* 
   TI_REQUIRE(M >= 0 && W > 0 && E > 0 && E <= MOE_MAX_EXPERTS && top > 0 && top <= E && top <= MOE_MAX_TOP,
              "moe_route: bad sizes M=%d W=%d experts=%d top=%d (up to %d experts, top up to %d)", M, W, E, top, MOE_MAX_EXPERTS,
              MOE_MAX_TOP);
-  TI_REQUIRE(score_kind == MOE_SIGMOID || score_kind == MOE_SOFTMAX, "moe_route: unknown score kind %d", score_kind);
+  TI_REQUIRE(score_kind == MOE_SIGMOID || score_kind == MOE_SOFTMAX || score_kind == MOE_SOFTMAX_CHOSEN, "moe_route: unknown score kind %d", score_kind);
   if (M == 0) return 0;
   const int piece = dtype == TI_F32 ? 4 : 8;
   const bool vec = W % piece == 0 && ((uintptr_t)h & 15) == 0;
@@ -232,10 +241,11 @@ __device__ __forceinline__ void wave_dots(const T* rows, int n_live, const T* __
 
 // DOWN false: rows are the tokens' inputs h (scaled by the score where it scales the input), K = W, outputs F, relu^2 to act.
 // DOWN true: rows are act, K = F, outputs W, 32-bit to part (times the score where it scales the output).
+// plain (DOWN false): the sums are stored as they are, in 32-bit (a gated activation over [gate | up] follows in a kernel of its own).
 template <typename T, bool VEC, int NP, bool DOWN>
 __global__ void __launch_bounds__(256)
 moe_expert_rows_kernel(const T* __restrict__ in, const int* __restrict__ ids, const float* __restrict__ wts, const T* __restrict__ w,
-                       void* __restrict__ out, int n_pairs, int K, int N, int top, int scale_input) {
+                       void* __restrict__ out, int n_pairs, int K, int N, int top, int scale_input, int plain) {
   extern __shared__ __attribute__((aligned(16))) unsigned char raw[];
   T* rows = reinterpret_cast<T*>(raw);      // [NP][K]
   __shared__ int s_pairs[NP], s_found[2];
@@ -270,6 +280,8 @@ moe_expert_rows_kernel(const T* __restrict__ in, const int* __restrict__ ids, co
               const int pair = s_pairs[p], n = n0 + r;
               if (DOWN) {
                 ((float*)out)[(size_t)pair * N + n] = scale_input ? z[r][p] : z[r][p] * wts[pair];
+              } else if (plain) {      // the sums themselves, 32-bit: an activation over several of them follows
+                ((float*)out)[(size_t)pair * N + n] = z[r][p];
               } else {
                 const float a = fmaxf(z[r][p], 0.f);
                 st<T>((T*)out + (size_t)pair * N + n, a * a);
@@ -293,18 +305,18 @@ __global__ void moe_sum_pairs_kernel(const float* __restrict__ part, float* __re
 
 template <typename T, bool VEC, int NP, bool DOWN>
 static void launch_expert_rows(const void* in, const int* ids, const float* wts, const void* w, void* out, int n_pairs, int K, int N,
-                               int top, int scale_input, int E, hipStream_t stream) {
+                               int top, int scale_input, int E, hipStream_t stream, int plain) {
   const dim3 grid(E, (N + 4 * MOE_ROWS - 1) / (4 * MOE_ROWS));
   moe_expert_rows_kernel<T, VEC, NP, DOWN><<<grid, 256, (size_t)NP * K * sizeof(T), stream>>>((const T*)in, ids, wts, (const T*)w, out,
-                                                                                               n_pairs, K, N, top, scale_input);
+                                                                                               n_pairs, K, N, top, scale_input, plain);
 }
 template <typename T, bool VEC, bool DOWN>
 static int expert_rows(const void* in, const int* ids, const float* wts, const void* w, void* out, int n_pairs, int K, int N, int top,
-                       int scale_input, int E, hipStream_t stream) {
+                       int scale_input, int E, hipStream_t stream, int plain = 0) {
   const size_t row = (size_t)K * sizeof(T), room = 48 * 1024;      // rows of the pairs a round holds in LDS
-  if (4 * row <= room) launch_expert_rows<T, VEC, 4, DOWN>(in, ids, wts, w, out, n_pairs, K, N, top, scale_input, E, stream);
-  else if (2 * row <= room) launch_expert_rows<T, VEC, 2, DOWN>(in, ids, wts, w, out, n_pairs, K, N, top, scale_input, E, stream);
-  else if (row <= 64 * 1024) launch_expert_rows<T, VEC, 1, DOWN>(in, ids, wts, w, out, n_pairs, K, N, top, scale_input, E, stream);
+  if (4 * row <= room) launch_expert_rows<T, VEC, 4, DOWN>(in, ids, wts, w, out, n_pairs, K, N, top, scale_input, E, stream, plain);
+  else if (2 * row <= room) launch_expert_rows<T, VEC, 2, DOWN>(in, ids, wts, w, out, n_pairs, K, N, top, scale_input, E, stream, plain);
+  else if (row <= 64 * 1024) launch_expert_rows<T, VEC, 1, DOWN>(in, ids, wts, w, out, n_pairs, K, N, top, scale_input, E, stream, plain);
   else return 1;
   return 0;
 }
@@ -338,6 +350,68 @@ extern "C" int ti_moe_experts_rows(int dtype, const void* h, const int* ids, con
     TI_REQUIRE(false, "moe_experts: unknown dtype %d", dtype);
   }
 #undef MOE_BOTH
+  TI_REQUIRE(rc == 0, "moe_experts: a row of %d or %d entries does not fit the workgroup's 64 KB", W, F);
+  if (y) moe_sum_pairs_kernel<<<M, 256, 0, stream>>>(part, y, W, top);
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------------------------------ gated experts
+// y[m] = sum_k s_k W_down[e_k] act(W_gate[e_k] h, W_up[e_k] h): gate_up [E][2F][W] holds an expert's gate rows above its up rows.
+//   act_kind 1: g = min(g, limit), u = clamp(u, -limit, limit); g * sigmoid(alpha g) * (u + 1)        0: silu(g) * u
+// z: f32 scratch [M top][2F] (the two products' sums), act: scratch of the dtype of h [M top][F], part: f32 [M top][W].
+template <typename T>
+__global__ void moe_gate_kernel(const float* __restrict__ z, T* __restrict__ act, long n_pairs, int F, int kind, float limit, float alpha) {
+  const long n = n_pairs * F;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+    const long pair = i / F;
+    const int f = (int)(i % F);
+    float g = z[pair * 2 * F + f], u = z[pair * 2 * F + F + f];
+    float y;
+    if (kind == 0) {
+      y = g / (1.0f + expf(-g)) * u;
+    } else {
+      g = fminf(g, limit);
+      u = fminf(fmaxf(u, -limit), limit);
+      y = g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
+    }
+    st<T>(act + i, y);
+  }
+}
+
+extern "C" int ti_moe_experts_rows_gated(int dtype, const void* h, const int* ids, const float* wts, const void* gate_up, const void* down,
+                                         float* z, void* act, float* part, float* y, int M, int W, int F, int E, int top, int act_kind,
+                                         float limit, float alpha, hipStream_t stream) {
+  TI_REQUIRE(M >= 0 && W > 0 && F > 0 && top > 0 && E > 0, "moe_experts: bad sizes M=%d W=%d F=%d top=%d", M, W, F, top);
+  TI_REQUIRE(act_kind == 0 || act_kind == 1, "moe_experts: unknown gated activation %d", act_kind);
+  if (M == 0) return 0;
+  TI_REQUIRE((2 * F + 4 * MOE_ROWS - 1) / (4 * MOE_ROWS) <= 65535 && (W + 4 * MOE_ROWS - 1) / (4 * MOE_ROWS) <= 65535,
+             "moe_experts: sizes W=%d F=%d are too large", W, F);
+  const int es = dtype == TI_F32 ? 4 : 2;
+  const int piece = 16 / es;
+  const bool vec = W % piece == 0 && F % piece == 0 && (((uintptr_t)gate_up | (uintptr_t)down | (uintptr_t)act | (uintptr_t)h) & 15) == 0;
+  const int n_pairs = M * top;
+  const long n_act = (long)n_pairs * F;
+  const unsigned blocks = (unsigned)((n_act + 255) / 256 < 16384 ? (n_act + 255) / 256 : 16384);
+  int rc;
+#define MOE_GATED(T, V)                                                                                                 \
+  do {                                                                                                                  \
+    rc = expert_rows<T, V, false>(h, ids, wts, gate_up, z, n_pairs, W, 2 * F, top, 0, E, stream, 1);                    \
+    if (rc == 0) {                                                                                                      \
+      moe_gate_kernel<T><<<blocks, 256, 0, stream>>>(z, (T*)act, n_pairs, F, act_kind, limit, alpha);                   \
+      rc = expert_rows<T, V, true>(act, ids, wts, down, part, n_pairs, F, W, top, 0, E, stream);                        \
+    }                                                                                                                   \
+  } while (0)
+  if (dtype == TI_F32) {
+    if (vec) MOE_GATED(float, true);
+    else MOE_GATED(float, false);
+  } else if (dtype == TI_BF16) {
+    if (vec) MOE_GATED(bf16_t, true);
+    else MOE_GATED(bf16_t, false);
+  } else {
+    TI_REQUIRE(false, "moe_experts: unknown dtype %d", dtype);
+  }
+#undef MOE_GATED
   TI_REQUIRE(rc == 0, "moe_experts: a row of %d or %d entries does not fit the workgroup's 64 KB", W, F);
   if (y) moe_sum_pairs_kernel<<<M, 256, 0, stream>>>(part, y, W, top);
   TI_LAUNCH_CHECK();

@@ -92,7 +92,7 @@ moe_place_kernel(const bf16_t* __restrict__ h, const int* __restrict__ ids, cons
   for (int i = 0; i < 16; ++i) {
     const int pair = pair0 + wave * 16 + i;
     if (pair >= n_pairs) break;
-    const float s = wts[pair];
+    const float s = wts ? wts[pair] : 1.f;      // no weights: the rows as they are (the weights come in at the end)
     const bf16_t* src = h + (size_t)(pair / top) * W;
     bf16_t* dst = rows + (size_t)s_row[wave * 16 + i] * W;
     for (int c = lane * 8; c < W; c += 64 * 8) {
@@ -227,6 +227,65 @@ extern "C" int ti_moe_experts_grouped_bf16(const void* h, const int* ids, const 
   moe_grouped_kernel<0><<<dim3(max_tiles, (F + 127) / 128), 256, 0, stream>>>((const bf16_t*)rows, (const bf16_t*)up, meta, E, act, F, W);
   moe_grouped_kernel<1><<<dim3(max_tiles, (W + 127) / 128), 256, 0, stream>>>((const bf16_t*)act, (const bf16_t*)down, meta, E, out, W, F);
   if (y) moe_combine_kernel<<<M, 256, 0, stream>>>(out, where, y, W, top);
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------------------------------ gated experts
+// out = sum_k s_k down_e act(gate_e h, up_e h) with gate_up [E][2F][W]: the rows are placed unscaled, one grouped product leaves
+// the sums of [gate | up] in 32-bit (z), the activation is taken in 32-bit and rounded once, the second grouped product
+// leaves a pair's row, and a token's rows are added times their weights in the order of choice.
+__global__ void moe_gate_rows_kernel(const float* __restrict__ z, bf16_t* __restrict__ act, long n_rows, int F, int kind, float limit,
+                                     float alpha) {
+  const long n = n_rows * F;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+    const long row = i / F;
+    const int f = (int)(i % F);
+    float g = z[row * 2 * F + f], u = z[row * 2 * F + F + f];
+    float y;
+    if (kind == 0) {
+      y = g / (1.0f + expf(-g)) * u;
+    } else {
+      g = fminf(g, limit);
+      u = fminf(fmaxf(u, -limit), limit);
+      y = g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
+    }
+    act[i] = f2bf(y);
+  }
+}
+
+// y[m] = sum_k wts[m top + k] out[where[m top + k]], k ascending
+__global__ void moe_combine_weighted_kernel(const float* __restrict__ out, const int* __restrict__ where, const float* __restrict__ wts,
+                                            float* __restrict__ y, int W, int top) {
+  const int m = blockIdx.x;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    float v = 0.f;
+    for (int k = 0; k < top; ++k) v = fmaf(wts[m * top + k], out[(size_t)where[m * top + k] * W + c], v);
+    y[(size_t)m * W + c] = v;
+  }
+}
+
+// Scratch as ti_moe_experts_grouped_bf16, and z f32 [M top][2F].  3: sizes not served (W, F multiples of 32, E <= 1024).
+extern "C" int ti_moe_experts_grouped_gated_bf16(const void* h, const int* ids, const float* wts, const void* gate_up, const void* down,
+                                                 int* meta, int* where, void* rows, float* z, void* act, float* out, float* y, int M,
+                                                 int W, int F, int E, int top, int act_kind, float limit, float alpha,
+                                                 hipStream_t stream) {
+  if (W % 32 || F % 32 || E > MOE_MAX_E) {
+    ti_set_error("moe_experts (grouped, gated): W=%d, F=%d, %d experts are not served", W, F, E);
+    return 3;
+  }
+  TI_REQUIRE(M >= 0 && top > 0 && E > 0 && y && (act_kind == 0 || act_kind == 1), "moe_experts (grouped, gated): bad arguments");
+  if (M == 0) return 0;
+  const int n_pairs = M * top;
+  const int max_tiles = (n_pairs + MOE_TILE - 1) / MOE_TILE + E;
+  moe_group_kernel<<<1, 1024, 0, stream>>>(ids, n_pairs, E, meta);
+  moe_place_kernel<<<(n_pairs + 63) / 64, 256, 0, stream>>>((const bf16_t*)h, ids, nullptr, meta, E, top, W, n_pairs, where, (bf16_t*)rows);
+  moe_grouped_kernel<1><<<dim3(max_tiles, (2 * F + 127) / 128), 256, 0, stream>>>((const bf16_t*)rows, (const bf16_t*)gate_up, meta, E, z, 2 * F, W);
+  const long n_act = (long)n_pairs * F;
+  const unsigned blocks = (unsigned)((n_act + 255) / 256 < 16384 ? (n_act + 255) / 256 : 16384);
+  moe_gate_rows_kernel<<<blocks, 256, 0, stream>>>(z, (bf16_t*)act, n_pairs, F, act_kind, limit, alpha);
+  moe_grouped_kernel<1><<<dim3(max_tiles, (W + 127) / 128), 256, 0, stream>>>((const bf16_t*)act, (const bf16_t*)down, meta, E, out, W, F);
+  moe_combine_weighted_kernel<<<M, 256, 0, stream>>>(out, where, wts, y, W, top);
   TI_LAUNCH_CHECK();
   return 0;
 }

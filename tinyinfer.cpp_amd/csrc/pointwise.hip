@@ -232,3 +232,182 @@ extern "C" int ti_qkv_split_write(int dtype, const float* qkv, const int* pos, c
   TI_LAUNCH_CHECK();
   return 0;
 }
+
+// ------------------------------------------------------------ q/k/v split with biases and a partial rotation
+// The same split with what a projection may still owe its rows: a bias on every column of qkv (null: none) and the
+// rotation of the first rot_dims entries of every query and key head (entry i with entry i + rot_dims / 2 by the angle
+// pos * inv_freq[i]; cosine and sine times mag; rope_table [table_len][rot_dims / 2][2] holds them ready for positions
+// below table_len; inv_freq null: none).  Bias and rotation happen in 32-bit, before the query's factor.
+__device__ __forceinline__ void rotation_of(const float* __restrict__ inv_freq, const float* __restrict__ rope_table, int table_len,
+                                            float mag, int half, int p, int i, float* c, float* s) {
+  if (rope_table && p < table_len) {
+    *c = rope_table[((size_t)p * half + i) * 2];
+    *s = rope_table[((size_t)p * half + i) * 2 + 1];
+  } else {
+    const float a = (float)p * inv_freq[i];
+    *c = cosf(a) * mag;
+    *s = sinf(a) * mag;
+  }
+}
+
+template <typename T>
+__global__ void qkv_prep_write_kernel(const float* __restrict__ qkv, const float* __restrict__ bias,
+                                      const float* __restrict__ inv_freq, const float* __restrict__ rope_table, int table_len,
+                                      float mag, int rot_dims, const int* __restrict__ pos, const int* __restrict__ slot,
+                                      const int* __restrict__ table, int table_stride, T* __restrict__ pool, T* __restrict__ q_out,
+                                      int n_head, int n_kv, int dk, int dv, int P, float coef, int every) {
+  const int m = blockIdx.x;
+  const int p = pos[m];
+  const int nq = n_head * dk, nk = n_kv * dk, nv = n_kv * dv;
+  const float* row = qkv + (size_t)m * (nq + nk + nv);
+  const float temp = (coef != 0.f && every > 0) ? 1.f + coef * logf((float)((p + 1) / every) + 1.f) : 1.f;
+  const int page = table[(size_t)slot[m] * table_stride + p / P];
+  const int r = p % P;
+  T* base = pool + (size_t)max(page, 0) * ((size_t)n_kv * P * (dk + dv));
+  const int half = inv_freq ? rot_dims / 2 : 0;
+  // queries and keys: a thread takes entry d of a head, and with it entry d + half where d is turned
+  for (int e = threadIdx.x; e < nq + nk; e += blockDim.x) {
+    const int d = e % dk;
+    if (d >= half && d < 2 * half) continue;      // written by the thread of its partner
+    const bool is_q = e < nq;
+    float u = row[e] + (bias ? bias[e] : 0.f);
+    float w = 0.f;
+    if (d < half) {
+      w = row[e + half] + (bias ? bias[e + half] : 0.f);
+      float c, s;
+      rotation_of(inv_freq, rope_table, table_len, mag, half, p, d, &c, &s);
+      const float a = u * c - w * s;
+      w = w * c + u * s;
+      u = a;
+    }
+    if (is_q) {
+      st<T>(q_out + (size_t)m * nq + e, u * temp);
+      if (d < half) st<T>(q_out + (size_t)m * nq + e + half, w * temp);
+    } else if (page >= 0) {      // the host reserves pages first; never write astray
+      const int h = (e - nq) / dk;
+      T* dst = base + ((size_t)h * P + r) * dk + d;
+      st<T>(dst, u);
+      if (d < half) st<T>(dst + half, w);
+    }
+  }
+  if (page < 0) return;
+  T* vbase = base + (size_t)n_kv * P * dk;
+  for (int e = threadIdx.x; e < nv; e += blockDim.x) {
+    const int h = e / dv, d = e % dv;
+    st<T>(vbase + ((size_t)h * dv + d) * P + r, row[nq + nk + e] + (bias ? bias[nq + nk + e] : 0.f));
+  }
+}
+
+extern "C" int ti_qkv_prep_write(int dtype, const float* qkv, const float* bias, const float* inv_freq, const float* rope_table,
+                                 int table_len, float mag, int rot_dims, const int* pos, const int* slot, const int* table,
+                                 int table_stride, void* pool, void* q_out, int M, int n_head, int n_kv, int dk, int dv,
+                                 int page_size, float coef, int every, hipStream_t stream) {
+  TI_REQUIRE(n_head > 0 && n_kv > 0 && dk > 0 && dv > 0 && page_size > 0 && table_stride > 0,
+             "qkv_prep_write: bad sizes heads=%d kv_heads=%d dk=%d dv=%d page=%d table_stride=%d", n_head, n_kv, dk, dv,
+             page_size, table_stride);
+  TI_REQUIRE(!inv_freq || (rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= dk),
+             "qkv_prep_write: %d rotated entries do not fit a head of %d (even, at most the head)", rot_dims, dk);
+  if (M == 0) return 0;
+  if (dtype == TI_F32)
+    qkv_prep_write_kernel<float><<<M, 256, 0, stream>>>(qkv, bias, inv_freq, rope_table, table_len, mag, rot_dims, pos, slot, table,
+                                                        table_stride, (float*)pool, (float*)q_out, n_head, n_kv, dk, dv,
+                                                        page_size, coef, every);
+  else if (dtype == TI_BF16)
+    qkv_prep_write_kernel<bf16_t><<<M, 256, 0, stream>>>(qkv, bias, inv_freq, rope_table, table_len, mag, rot_dims, pos, slot, table,
+                                                         table_stride, (bf16_t*)pool, (bf16_t*)q_out, n_head, n_kv, dk, dv,
+                                                         page_size, coef, every);
+  else
+    TI_REQUIRE(false, "qkv_prep_write: unknown dtype %d", dtype);
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------------------------------ Dynamic Tanh
+// out[r, c] = tanh(alpha x[rows ? rows[r] : r, c]) * w[c] + b[c]: a norm that takes no mean and no variance.  alpha is one
+// learned number (device memory).  32-bit arithmetic, rounded once to T.
+template <typename T>
+__global__ void dyt_kernel(const float* __restrict__ x, const float* __restrict__ alpha, const float* __restrict__ w,
+                           const float* __restrict__ b, const int* __restrict__ rows, T* __restrict__ out, int H) {
+  const int r = blockIdx.x;
+  const float a = alpha[0];
+  const float* src = x + (size_t)(rows ? rows[r] : r) * H;
+  for (int c = threadIdx.x; c < H; c += blockDim.x) st<T>(out + (size_t)r * H + c, fmaf(tanhf(a * src[c]), w[c], b ? b[c] : 0.f));
+}
+
+extern "C" int ti_dyt(int out_dtype, const float* x, const float* alpha, const float* w, const float* b, const int* rows, void* out,
+                      int n_rows, int H, hipStream_t stream) {
+  TI_REQUIRE(n_rows >= 0 && H > 0 && alpha && w, "dyt: bad sizes rows=%d H=%d", n_rows, H);
+  if (n_rows == 0) return 0;
+  if (out_dtype == TI_F32) dyt_kernel<float><<<n_rows, 256, 0, stream>>>(x, alpha, w, b, rows, (float*)out, H);
+  else if (out_dtype == TI_BF16) dyt_kernel<bf16_t><<<n_rows, 256, 0, stream>>>(x, alpha, w, b, rows, (bf16_t*)out, H);
+  else TI_REQUIRE(false, "dyt: unknown dtype %d", out_dtype);
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------------------------------ gated activations between a feed-forward's products
+// z f32 [R, 2F] = [gate | up] (rows ldz floats apart), bias f32 [2F] (null: none) added first.
+//   kind 0: out = silu(g) * u
+//   kind 1: g = min(g, limit), u = clamp(u, -limit, limit); out = g * sigmoid(alpha g) * (u + 1)
+__device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
+
+template <typename T>
+__global__ void gated_act_kernel(const float* __restrict__ z, long ldz, const float* __restrict__ bias, T* __restrict__ out, long R,
+                                 int F, int kind, float limit, float alpha) {
+  const long n = R * F;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+    const long r = i / F;
+    const int f = (int)(i % F);
+    float g = z[r * ldz + f], u = z[r * ldz + F + f];
+    if (bias) {
+      g += bias[f];
+      u += bias[F + f];
+    }
+    float y;
+    if (kind == 0) {
+      y = g * sigmoid_f(g) * u;
+    } else {
+      g = fminf(g, limit);
+      u = fminf(fmaxf(u, -limit), limit);
+      y = g * sigmoid_f(alpha * g) * (u + 1.0f);
+    }
+    st<T>(out + i, y);
+  }
+}
+
+extern "C" int ti_gated_act(int out_dtype, const float* z, long ldz, const float* bias, void* out, long R, int F, int kind,
+                            float limit, float alpha, hipStream_t stream) {
+  TI_REQUIRE(R >= 0 && F > 0 && ldz >= 2L * F && (kind == 0 || kind == 1), "gated_act: bad sizes R=%ld F=%d ld=%ld kind=%d", R, F, ldz, kind);
+  if (R == 0) return 0;
+  const long n = R * F;
+  const unsigned blocks = (unsigned)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
+  if (out_dtype == TI_F32) gated_act_kernel<float><<<blocks, 256, 0, stream>>>(z, ldz, bias, (float*)out, R, F, kind, limit, alpha);
+  else if (out_dtype == TI_BF16) gated_act_kernel<bf16_t><<<blocks, 256, 0, stream>>>(z, ldz, bias, (bf16_t*)out, R, F, kind, limit, alpha);
+  else TI_REQUIRE(false, "gated_act: unknown dtype %d", out_dtype);
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------------------------------ two streams side by side, rounded
+// out T [M, 2H] = [a | b] for the product that mixes the residual with a stream kept from earlier in the step
+template <typename T>
+__global__ void concat_round_kernel(const float* __restrict__ a, const float* __restrict__ b, T* __restrict__ out, long M, int H) {
+  const long n = M * 2 * H;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+    const long m = i / (2 * H);
+    const int c = (int)(i % (2 * H));
+    st<T>(out + i, c < H ? a[m * H + c] : b[m * H + c - H]);
+  }
+}
+
+extern "C" int ti_concat_round(int out_dtype, const float* a, const float* b, void* out, int M, int H, hipStream_t stream) {
+  TI_REQUIRE(M >= 0 && H > 0, "concat_round: bad sizes M=%d H=%d", M, H);
+  if (M == 0) return 0;
+  const long n = (long)M * 2 * H;
+  const unsigned blocks = (unsigned)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
+  if (out_dtype == TI_F32) concat_round_kernel<float><<<blocks, 256, 0, stream>>>(a, b, (float*)out, M, H);
+  else if (out_dtype == TI_BF16) concat_round_kernel<bf16_t><<<blocks, 256, 0, stream>>>(a, b, (bf16_t*)out, M, H);
+  else TI_REQUIRE(false, "concat_round: unknown dtype %d", out_dtype);
+  TI_LAUNCH_CHECK();
+  return 0;
+}

@@ -114,6 +114,43 @@ int ti_qkv_split_write(int dtype, const float* qkv, const int* pos, const int* s
                        void* pool, void* q_out, int M, int n_head, int n_kv, int dk, int dv, int page_size, float coef,
                        int every, hipStream_t stream);
 
+// the same split with a bias on every column of qkv first (f32 [n_head dk + n_kv (dk + dv)], null: none) and the rotation of
+// the first rot_dims entries of every query and key head (entry i with entry i + rot_dims / 2; cos and sin times mag;
+// rope_table [table_len][rot_dims / 2][2] may be null; inv_freq null: no rotation)
+int ti_qkv_prep_write(int dtype, const float* qkv, const float* bias, const float* inv_freq, const float* rope_table,
+                      int table_len, float mag, int rot_dims, const int* pos, const int* slot, const int* table,
+                      int table_stride, void* pool, void* q_out, int M, int n_head, int n_kv, int dk, int dv, int page_size,
+                      float coef, int every, hipStream_t stream);
+// out[r] = tanh(alpha[0] x[rows ? rows[r] : r]) * w + b (b may be null), in `out_dtype`
+int ti_dyt(int out_dtype, const float* x, const float* alpha, const float* w, const float* b, const int* rows, void* out,
+           int n_rows, int H, hipStream_t stream);
+// z f32 [R, 2F] = [gate | up], rows ldz floats apart, bias f32 [2F] (null: none) added first.  kind 0: silu(g) u;
+// kind 1: g = min(g, limit), u = clamp(u, -limit, limit), g sigmoid(alpha g) (u + 1).  out [R, F] in `out_dtype`
+int ti_gated_act(int out_dtype, const float* z, long ldz, const float* bias, void* out, long R, int F, int kind, float limit,
+                 float alpha, hipStream_t stream);
+// out [M, 2H] = [a | b] rounded to `out_dtype` (a, b f32 [M, H])
+int ti_concat_round(int out_dtype, const float* a, const float* b, void* out, int M, int H, hipStream_t stream);
+
+// ---- libti_latent_attention: attention over cached latents (a token keeps [c (R) | kr (r)]; a head's key is [W_uk c | kr],
+// its value W_uv c, neither ever formed per token)
+// proj f32 [M, ld]: queries [H][d + r] from column 0, [latent (R) | shared key part (r)] from column off_kv.  The latent is
+// RMS-normed (norm_w [R], eps) and goes with the rotated key part into the token's row of pool [pages][P][R + r]; the heads'
+// last r query entries are rotated in place.  Rotation as in ti_qkv_prep_write (rot_dims <= r)
+int ti_latent_prep(int dtype, float* proj, int ld, int off_kv, const float* norm_w, float eps, const float* inv_freq,
+                   const float* rope_table, int table_len, float mag, int rot_dims, const int* pos, const int* slot,
+                   const int* table, int table_stride, void* pool, int M, int H, int d, int r, int R, int page_size,
+                   hipStream_t stream);
+// qa f32 [M, H, R + r] = [W_uk_h^T q_h[:d] | q_h[d:]] with w_uk [H d][R] in `dtype`
+int ti_latent_absorb(int dtype, const float* proj, int ld, const void* w_uk, float* qa, int M, int H, int d, int r, int R,
+                     hipStream_t stream);
+// o f32 [M, H, R] = sum_j p_j c_j over the row's visible positions (window <= 0: all up to its own), p the softmax of
+// (qa . [c_j | kr_j]) scale with exp(sink[h]) joining the denominator (sink null: none)
+int ti_latent_attention_rows(int dtype, const float* qa, const void* pool, const int* table, int table_stride, const int* pos,
+                             const int* slot, const float* sink, float* out, int M, int H, int R, int r, int page_size,
+                             float scale, int window, hipStream_t stream);
+// out [M, H dv] = W_uv_h o[m, h] with w_uv [H dv][R], both in `dtype`
+int ti_latent_expand(int dtype, const float* o, const void* w_uv, void* out, int M, int H, int R, int dv, hipStream_t stream);
+
 // ---- libti_recurrent: the mLSTM cell as a scan over each request's tokens of the step
 // proj f32 [M, ld] holds, from the columns off_* on, the heads' q and k [heads][dk], v [heads][dv] and the gates'
 // pre-activations i, f [heads]; state f32, slot_stride floats per slot: [heads][dk dv + dk + 1] (S [dk][dv], n, m);
@@ -184,7 +221,8 @@ int ti_diff_attention_rows_bf16(const void* q, const void* pool, const int* tabl
 long ti_diff_attention_rows_scratch(int n_rows, int n_kv, int dv, int n_splits);
 
 // ---- libti_moe: a mixture of experts
-// scores (score_kind 0: sigmoid, 1: softmax over the experts) of h [M, W] against router f32 [E, W] in 32-bit; the `top`
+// scores (score_kind 0: sigmoid, 1: softmax over the experts, 2: the logits themselves, the weights then being the softmax over
+// the chosen logits alone) of h [M, W] against router f32 [E, W] in 32-bit; the `top`
 // largest per token (ties: the lower index) to ids int32 [M, top] and wts f32 [M, top] (renormalize: divided by their sum)
 int ti_moe_route(int dtype, const void* h, const float* router, int* ids, float* wts, int M, int W, int E, int top,
                  int score_kind, int renormalize, hipStream_t stream);
@@ -195,6 +233,13 @@ int ti_moe_route(int dtype, const void* h, const float* router, int* ids, float*
 int ti_moe_experts_rows(int dtype, const void* h, const int* ids, const float* wts, const void* up, const void* down, void* act,
                         float* part, float* y, int M, int W, int F, int E, int top, int scale_input, hipStream_t stream);
 
+// experts with a gate: y[m] = sum_k s_k down[e_k] act(gate[e_k] h, up[e_k] h); gate_up [E][2F][W] holds an expert's gate rows
+// above its up rows.  act_kind 0: silu(g) u; 1: g = min(g, limit), u = clamp(u, -limit, limit), g sigmoid(alpha g) (u + 1).
+// z: f32 scratch [M top][2F]; act, part, y as above
+int ti_moe_experts_rows_gated(int dtype, const void* h, const int* ids, const float* wts, const void* gate_up, const void* down,
+                              float* z, void* act, float* part, float* y, int M, int W, int F, int E, int top, int act_kind,
+                              float limit, float alpha, hipStream_t stream);
+
 // ---- libti_moe_bf16: the experts for steps of many tokens, on the matrix cores: the (token, expert) pairs are laid out expert
 // by expert in tiles of 128 rows and both products run over the tiles.  Scratch: meta int32 [ti_moe_grouped_meta_ints(M top, E)],
 // where int32 [M top] (the row of every pair), rows bf16 [M top][W], act bf16 [M top][F], out f32 [M top][W].  y (may be
@@ -203,6 +248,11 @@ long ti_moe_grouped_meta_ints(int n_pairs, int E);
 int ti_moe_experts_grouped_bf16(const void* h, const int* ids, const float* wts, const void* up, const void* down, int* meta,
                                 int* where, void* rows, void* act, float* out, float* y, int M, int W, int F, int E, int top,
                                 int scale_input, hipStream_t stream);
+
+// the gated experts of ti_moe_experts_rows_gated over such tiles; z: f32 scratch [M top][2F]; y is written (the tokens' weighted sums)
+int ti_moe_experts_grouped_gated_bf16(const void* h, const int* ids, const float* wts, const void* gate_up, const void* down,
+                                      int* meta, int* where, void* rows, float* z, void* act, float* out, float* y, int M, int W,
+                                      int F, int E, int top, int act_kind, float limit, float alpha, hipStream_t stream);
 
 // ---- libti_attention_bf16: the same on the matrix cores (head sizes 32, 64, 128; pages of 16 n rows)
 // rows of single tokens; n_splits > 1 needs part_o f32 [n_rows, n_head, n_splits, hd] and part_ml f32

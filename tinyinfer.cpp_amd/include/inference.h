@@ -166,6 +166,9 @@ ModelSpec miterax_spec(const Json& config);
 // the Mumasun decoder (config/mumasun.cpp)
 Json mumasun_typed_config(const Json& config);
 ModelSpec mumasun_spec(const Json& config);
+// the Nazorax decoder (config/nazorax.cpp)
+Json nazorax_typed_config(const Json& config);
+ModelSpec nazorax_spec(const Json& config);
 // {"architecture": the registered name that matched, "config": the typed configuration (the input itself if
 // the architecture registered no reader)}; ConfigError as spec_from_config
 Json typed_config(const Json& config);
@@ -334,6 +337,11 @@ class Ops {
   // 1 + coef ln(floor((pos + 1) / every) + 1) to q_out, k and v into the pages (K [kv][P][dk] | V [kv][dv][P])
   void qkv_split_write(const Tensor& qkv, const int* positions, const int* slots, const CacheView& view, const Tensor& pool,
                        const Tensor& q_out, int heads, int kv_heads, int dk, int dv, float temp_coef, int temp_every);
+  // the same split with what the projection still owes its rows: a bias on every column (f32 [width], undefined: none) and the
+  // rotation `rot` of the leading entries of every query and key head (rot.inv_freq null: none), both in 32-bit
+  void qkv_split_write(const Tensor& qkv, const Tensor& bias, const Rotation& rot, const int* positions, const int* slots,
+                       const CacheView& view, const Tensor& pool, const Tensor& q_out, int heads, int kv_heads, int dk, int dv,
+                       float temp_coef, int temp_every);
   // causal attention of every row over such pages, scores soft-capped: softcap tanh(s / softcap) (softcap 0: none)
   void attention_capped(const Tensor& q, const Tensor& pool, const CacheView& view, const int* positions, const int* slots,
                         const Tensor& out, int heads, int kv_heads, int dk, int dv, float scale, float softcap, int window);
@@ -348,6 +356,26 @@ class Ops {
   // out = o / rms(o per head) * w * sigmoid(gate columns of proj), in the compute dtype
   void gated_head_norm(const Tensor& o, const Tensor& proj, int gate_col, const Tensor& w, float eps, const Tensor& out,
                        int heads, int dv);
+  // ---- Dynamic Tanh, gated feed-forwards with biases, latent attention, a stream kept for later
+  // out[r] = tanh(alpha x[rows ? rows[r] : r]) * w + b: alpha f32 [1], b may be undefined
+  void dyt(const Tensor& x, const Tensor& alpha, const Tensor& w, const Tensor& b, const Tensor& out, const int* rows = nullptr,
+           int64_t n_rows = 0);
+  // z f32 [R, 2F] = [gate | up] (+ bias f32 [2F], may be undefined) -> out [R, F] in its own dtype
+  enum GatedAct { Silu = 0, ClampedGlu = 1 };   // silu(g) u;  g = min(g, limit), u = clamp(u, -limit, limit): g sigmoid(alpha g) (u + 1)
+  void gated_act(const Tensor& z, const Tensor& bias, const Tensor& out, GatedAct kind, float limit = 0.f, float alpha = 1.f);
+  // out [M, 2H] = [a | b] in out's dtype
+  void concat_round(const Tensor& a, const Tensor& b, const Tensor& out);
+  // Latent attention (a token keeps a normed latent of `rank` numbers and one rotated key part of `rot_dim`, pool
+  // [pages][P][rank + rot_dim]; a head's key is [W_uk c | kr], its value W_uv c).  proj f32 [M, >= off_kv + rank + rot_dim]:
+  // the heads' queries [heads][dim + rot_dim] from column 0, latent and key part from column off_kv.
+  // latent_prep: the latent normed (norm_w, eps) and the key part rotated into the token's row; the heads' rotated parts turned in place
+  void latent_prep(const Tensor& proj, int off_kv, const Tensor& norm_w, float eps, const Rotation& rot, const int* positions,
+                   const int* slots, const CacheView& view, const Tensor& pool, int heads, int dim, int rot_dim, int rank);
+  // out [M, heads v_dim] = W_uv (softmax((W_uk^T q | q_rot) . [c | kr] scale; sink) c): scores and softmax in 32-bit, the
+  // sink (f32 [heads], may be undefined) in the denominator only; scratch from `ws`
+  void latent_attention(const Tensor& proj, const Tensor& w_uk, const Tensor& w_uv, const Tensor& sink, const Tensor& pool,
+                        const CacheView& view, const int* positions, const int* slots, const Tensor& out, int heads, int dim,
+                        int rot_dim, int rank, int v_dim, float scale, int window, Workspace& ws);
   // ---- layers that norm what a sublayer returns; short convolutions; differential attention; mixtures of experts
   // x (+)= y / rms(y) * gain (32-bit; gain is the factor itself).  accumulate false: x is overwritten (y may be x).
   // gather (device int32 [M][n_gather]): row m of y is the sum of the rows y[gather[m][k]], k ascending; no list and
@@ -380,7 +408,7 @@ class Ops {
   void diff_attention(const Tensor& q, const Tensor& pool, const CacheView& view, const int* positions, const int* slots,
                       const Tensor& out, int heads, int kv_heads, int dk, int dv, float scale, int block, int window, float lambda,
                       float eps, float out_scale, const DiffAttentionLists* lists = nullptr);
-  enum RouterScore { Sigmoid = 0, Softmax = 1 };
+  enum RouterScore { Sigmoid = 0, Softmax = 1, SoftmaxChosen = 2 };   // 2: the largest logits chosen, weights = softmax over them alone
   // the `top` experts with the largest scores of h against router f32 [E, W]: ids int32 [M, top], wts f32 [M, top]
   void moe_route(const Tensor& h, const Tensor& router, const Tensor& ids, const Tensor& wts, int top, RouterScore score,
                  bool renormalize);
@@ -392,6 +420,10 @@ class Ops {
   struct GatheredRows { Tensor t; const int* gather = nullptr; int n_gather = 0; };
   void moe_experts(const Tensor& h, const Tensor& ids, const Tensor& wts, const Tensor& up, const Tensor& down, const Tensor& y,
                    int experts, bool scale_input, Workspace& ws, GatheredRows* rows = nullptr);
+  // experts with a gate: y = sum_k s_k down_e act(gate_e h, up_e h); gate_up [E 2F, W] holds an expert's gate rows above its up rows
+  void moe_experts_gated(const Tensor& h, const Tensor& ids, const Tensor& wts, const Tensor& gate_up, const Tensor& down,
+                         const Tensor& y, int experts, GatedAct kind, float limit, float alpha, Workspace& ws,
+                         GatheredRows* rows = nullptr);
   void argmax(const Tensor& logits, int* out);
   void sample(const Tensor& logits, const float* temperature, const int* top_k, const float* top_p, const float* uniform,
               int* out);

@@ -924,6 +924,121 @@ void Ops::qkv_split_write(const Tensor& qkv, const int* positions, const int* sl
   check("pointwise", rc, "qkv_split_write");
 }
 
+void Ops::qkv_split_write(const Tensor& qkv, const Tensor& bias, const Rotation& rot, const int* positions, const int* slots,
+                          const CacheView& view, const Tensor& pool, const Tensor& q_out, int heads, int kv_heads, int dk, int dv,
+                          float temp_coef, int temp_every) {
+  TIMED("qkv_split_write " + dims(qkv) + (bias.defined() ? " bias" : "") + (rot.inv_freq ? " rotation" : ""));
+  const int64_t M = qkv.shape[0];
+  const int64_t width = (int64_t)heads * dk + (int64_t)kv_heads * (dk + dv);
+  require(qkv.ndim == 2 && qkv.shape[1] == width && qkv.dtype == DType::F32 && qkv.contiguous(),
+          "qkv_split_write: qkv " + qkv.describe() + " does not fit [M, " + std::to_string(width) + "] float32");
+  require(!bias.defined() || (bias.dtype == DType::F32 && bias.numel() == width && bias.contiguous()),
+          "qkv_split_write: bias " + bias.describe() + " does not fit float32 [" + std::to_string(width) + "]");
+  require(q_out.ndim == 2 && q_out.shape[0] == M && q_out.shape[1] == (int64_t)heads * dk && q_out.contiguous(),
+          "qkv_split_write: q_out has the wrong shape");
+  check_split_pool("qkv_split_write", pool, kv_heads, dk, dv, q_out.dtype);
+  const int rot_dims = rot.inv_freq ? (rot.dims > 0 ? rot.dims : dk) : 0;
+  require(rot_dims % 2 == 0 && rot_dims <= dk, "qkv_split_write: " + std::to_string(rot_dims) + " rotated entries do not fit a head of " + std::to_string(dk));
+  int rc = KERNEL("pointwise", ti_qkv_prep_write)(code(q_out.dtype, "qkv_split_write"), (const float*)qkv.data,
+                                                  bias.defined() ? (const float*)bias.data : nullptr, rot.inv_freq, rot.table,
+                                                  rot.table_len, rot.mag, rot_dims, positions, slots, view.table, view.table_width,
+                                                  pool.data, q_out.data, (int)M, heads, kv_heads, dk, dv, (int)pool.shape[2],
+                                                  temp_coef, temp_every, (hipStream_t)launch_stream());
+  check("pointwise", rc, "qkv_split_write");
+}
+
+void Ops::dyt(const Tensor& x, const Tensor& alpha, const Tensor& w, const Tensor& b, const Tensor& out, const int* rows, int64_t n_rows) {
+  TIMED("dyt " + std::to_string(rows ? n_rows : x.shape[0]) + "x" + std::to_string(x.shape[1]));
+  require(x.ndim == 2 && x.dtype == DType::F32 && x.contiguous(), "dyt: x must be a contiguous float32 matrix");
+  const int64_t H = x.shape[1], n = rows ? n_rows : x.shape[0];
+  require(alpha.dtype == DType::F32 && alpha.numel() == 1 && w.dtype == DType::F32 && w.numel() == H &&
+              (!b.defined() || (b.dtype == DType::F32 && b.numel() == H)),
+          "dyt: alpha " + alpha.describe() + ", w " + w.describe() + " or b " + b.describe() + " do not fit width " + std::to_string(H));
+  require(out.ndim == 2 && out.shape[0] == n && out.shape[1] == H && out.contiguous(), "dyt: out " + out.describe() + " does not fit");
+  int rc = KERNEL("pointwise", ti_dyt)(code(out.dtype, "dyt"), (const float*)x.data, (const float*)alpha.data, (const float*)w.data,
+                                       b.defined() ? (const float*)b.data : nullptr, rows, out.data, (int)n, (int)H,
+                                       (hipStream_t)launch_stream());
+  check("pointwise", rc, "dyt");
+}
+
+void Ops::gated_act(const Tensor& z, const Tensor& bias, const Tensor& out, GatedAct kind, float limit, float alpha) {
+  TIMED("gated_act " + dims(z));
+  require(z.ndim == 2 && z.dtype == DType::F32 && z.stride[1] == 1 && z.shape[1] % 2 == 0, "gated_act: z " + z.describe() + " must be float32 [R, 2F]");
+  const int64_t R = z.shape[0], F = z.shape[1] / 2;
+  require(!bias.defined() || (bias.dtype == DType::F32 && bias.numel() == 2 * F), "gated_act: bias " + bias.describe() + " does not fit [2F]");
+  require(out.ndim == 2 && out.shape[0] == R && out.shape[1] == F && out.contiguous(), "gated_act: out " + out.describe() + " does not fit [R, F]");
+  int rc = KERNEL("pointwise", ti_gated_act)(code(out.dtype, "gated_act"), (const float*)z.data, (long)z.stride[0],
+                                             bias.defined() ? (const float*)bias.data : nullptr, out.data, (long)R, (int)F, (int)kind,
+                                             limit, alpha, (hipStream_t)launch_stream());
+  check("pointwise", rc, "gated_act");
+}
+
+void Ops::concat_round(const Tensor& a, const Tensor& b, const Tensor& out) {
+  TIMED("concat_round " + dims(a));
+  require(a.ndim == 2 && a.dtype == DType::F32 && a.contiguous() && b.ndim == 2 && b.dtype == DType::F32 && b.contiguous() &&
+              b.shape[0] == a.shape[0] && b.shape[1] == a.shape[1] && out.ndim == 2 && out.shape[0] == a.shape[0] &&
+              out.shape[1] == 2 * a.shape[1] && out.contiguous(),
+          "concat_round: a " + a.describe() + ", b " + b.describe() + " and out " + out.describe() + " do not fit");
+  int rc = KERNEL("pointwise", ti_concat_round)(code(out.dtype, "concat_round"), (const float*)a.data, (const float*)b.data, out.data,
+                                                (int)a.shape[0], (int)a.shape[1], (hipStream_t)launch_stream());
+  check("pointwise", rc, "concat_round");
+}
+
+static void check_latent_pool(const char* what, const Tensor& pool, int rank, int rot_dim, DType dt) {
+  require(pool.ndim == 3 && pool.shape[2] == (int64_t)rank + rot_dim && pool.dtype == dt && pool.contiguous(),
+          std::string(what) + ": pool " + pool.describe() + " does not fit [pages, P, " + std::to_string(rank + rot_dim) + "] of " + dtype_name(dt));
+}
+
+void Ops::latent_prep(const Tensor& proj, int off_kv, const Tensor& norm_w, float eps, const Rotation& rot, const int* positions,
+                      const int* slots, const CacheView& view, const Tensor& pool, int heads, int dim, int rot_dim, int rank) {
+  TIMED("latent_prep " + dims(proj));
+  require(proj.ndim == 2 && proj.dtype == DType::F32 && proj.contiguous() && off_kv >= (int64_t)heads * (dim + rot_dim) &&
+              proj.shape[1] >= (int64_t)off_kv + rank + rot_dim,
+          "latent_prep: proj " + proj.describe() + " does not hold the queries and the latent");
+  require(norm_w.dtype == DType::F32 && norm_w.numel() == rank, "latent_prep: the latent's norm weight " + norm_w.describe() + " does not fit");
+  require(pool.ndim == 3 && pool.shape[2] == (int64_t)rank + rot_dim && pool.contiguous(), "latent_prep: pool " + pool.describe() + " does not fit");
+  const int rot_dims = rot.inv_freq ? (rot.dims > 0 ? rot.dims : rot_dim) : 0;
+  require(rot_dims % 2 == 0 && rot_dims <= rot_dim, "latent_prep: " + std::to_string(rot_dims) + " rotated entries do not fit " + std::to_string(rot_dim));
+  int rc = KERNEL("latent_attention", ti_latent_prep)(code(pool.dtype, "latent_prep"), (float*)proj.data, (int)proj.shape[1], off_kv,
+                                                      (const float*)norm_w.data, eps, rot.inv_freq, rot.table, rot.table_len, rot.mag,
+                                                      rot_dims, positions, slots, view.table, view.table_width, pool.data,
+                                                      (int)proj.shape[0], heads, dim, rot_dim, rank, (int)pool.shape[1],
+                                                      (hipStream_t)launch_stream());
+  check("latent_attention", rc, "latent_prep");
+}
+
+void Ops::latent_attention(const Tensor& proj, const Tensor& w_uk, const Tensor& w_uv, const Tensor& sink, const Tensor& pool,
+                           const CacheView& view, const int* positions, const int* slots, const Tensor& out, int heads, int dim,
+                           int rot_dim, int rank, int v_dim, float scale, int window, Workspace& ws) {
+  TIMED("latent_attention " + dims(proj));
+  const int64_t M = proj.shape[0];
+  require(proj.ndim == 2 && proj.dtype == DType::F32 && proj.contiguous() && proj.shape[1] >= (int64_t)heads * (dim + rot_dim),
+          "latent_attention: proj " + proj.describe() + " does not hold the queries");
+  check_latent_pool("latent_attention", pool, rank, rot_dim, out.dtype);
+  require(w_uk.ndim == 2 && w_uk.shape[0] == (int64_t)heads * dim && w_uk.shape[1] == rank && w_uk.contiguous() && w_uk.dtype == out.dtype &&
+              w_uv.ndim == 2 && w_uv.shape[0] == (int64_t)heads * v_dim && w_uv.shape[1] == rank && w_uv.contiguous() && w_uv.dtype == out.dtype,
+          "latent_attention: w_uk " + w_uk.describe() + " / w_uv " + w_uv.describe() + " do not fit");
+  require(!sink.defined() || (sink.dtype == DType::F32 && sink.numel() == heads), "latent_attention: sink " + sink.describe() + " does not fit [heads]");
+  require(out.ndim == 2 && out.shape[0] == M && out.shape[1] == (int64_t)heads * v_dim && out.contiguous(), "latent_attention: out has the wrong shape");
+  if (M == 0) return;
+  const int dt = code(out.dtype, "latent_attention");
+  Tensor qa = ws.tensor("latent.qa", DType::F32, {M, (int64_t)heads * (rank + rot_dim)});
+  Tensor o = ws.tensor("latent.o", DType::F32, {M, (int64_t)heads * rank});
+  void* stream = launch_stream();
+  int rc = KERNEL("latent_attention", ti_latent_absorb)(dt, (const float*)proj.data, (int)proj.shape[1], w_uk.data, (float*)qa.data, (int)M,
+                                                        heads, dim, rot_dim, rank, (hipStream_t)stream);
+  check("latent_attention", rc, "latent_attention(absorb)");
+  rc = KERNEL("latent_attention", ti_latent_attention_rows)(dt, (const float*)qa.data, pool.data, view.table, view.table_width, positions,
+                                                            slots, sink.defined() ? (const float*)sink.data : nullptr, (float*)o.data,
+                                                            (int)M, heads, rank, rot_dim, (int)pool.shape[1], scale, window,
+                                                            (hipStream_t)stream);
+  check("latent_attention", rc, "latent_attention(rows)");
+  took("[generic]");
+  rc = KERNEL("latent_attention", ti_latent_expand)(dt, (const float*)o.data, w_uv.data, out.data, (int)M, heads, rank, v_dim,
+                                                    (hipStream_t)stream);
+  check("latent_attention", rc, "latent_attention(expand)");
+}
+
 void Ops::attention_capped(const Tensor& q, const Tensor& pool, const CacheView& view, const int* positions, const int* slots,
                            const Tensor& out, int heads, int kv_heads, int dk, int dv, float scale, float softcap, int window) {
   TIMED("attention_capped " + dims(q));
@@ -1198,6 +1313,59 @@ void Ops::moe_experts(const Tensor& h, const Tensor& ids, const Tensor& wts, con
                                               up.data, down.data, act.data, (float*)part.data, (top == 1 || left) ? nullptr : (float*)y.data,
                                               (int)M, (int)W, (int)F, experts, top, scale_input ? 1 : 0, (hipStream_t)launch_stream());
   check("moe", rc, "moe_experts");
+  if (left) {
+    rows->t = part;
+    rows->gather = nullptr;
+    rows->n_gather = top;
+  }
+}
+
+void Ops::moe_experts_gated(const Tensor& h, const Tensor& ids, const Tensor& wts, const Tensor& gate_up, const Tensor& down,
+                            const Tensor& y, int experts, GatedAct kind, float limit, float alpha, Workspace& ws, GatheredRows* rows) {
+  TIMED("moe_experts_gated " + dims(h) + " * " + dims(gate_up));
+  require(h.ndim == 2 && h.contiguous() && gate_up.ndim == 2 && down.ndim == 2 && gate_up.contiguous() && down.contiguous() &&
+              gate_up.dtype == h.dtype && down.dtype == h.dtype && experts > 0,
+          "moe_experts_gated: h, gate_up and down must be matrices of one dtype");
+  const int64_t M = h.shape[0], W = h.shape[1];
+  require(gate_up.shape[1] == W && gate_up.shape[0] % (2 * experts) == 0, "moe_experts_gated: gate_up " + gate_up.describe() + " does not fit");
+  const int64_t F = gate_up.shape[0] / (2 * experts);
+  require(down.shape[0] == (int64_t)experts * W && down.shape[1] == F, "moe_experts_gated: down " + down.describe() + " does not fit");
+  require(y.ndim == 2 && y.dtype == DType::F32 && y.contiguous() && y.shape[0] == M && y.shape[1] == W,
+          "moe_experts_gated: y " + y.describe() + " does not fit");
+  require(ids.dtype == DType::I32 && wts.dtype == DType::F32 && ids.numel() == wts.numel() && (M == 0 || ids.numel() % M == 0),
+          "moe_experts_gated: ids and wts must be int32 / float32 [M, top]");
+  if (rows) *rows = GatheredRows();
+  if (M == 0) return;
+  const int top = (int)(ids.numel() / M);
+  const int64_t pairs = M * top;
+  Tensor z = ws.tensor("moe.z", DType::F32, {pairs, 2 * F});
+  // many tokens: the pairs grouped by expert, both products on the matrix cores
+  if (h.dtype == DType::BF16 && use.fast_gemm && pairs >= 128 && kernel_library_available("moe_bf16")) {
+    const long meta_ints = KERNEL("moe_bf16", ti_moe_grouped_meta_ints)((int)pairs, experts);
+    int* meta = (int*)ws.get("moe.meta", (size_t)meta_ints * 4);
+    Tensor where = ws.tensor("moe.where", DType::I32, {pairs});
+    Tensor sorted = ws.tensor("moe.rows", DType::BF16, {pairs, W});
+    Tensor act = ws.tensor("moe.act", DType::BF16, {pairs, F});
+    Tensor out = ws.tensor("moe.out", DType::F32, {pairs, W});
+    int rc = KERNEL("moe_bf16", ti_moe_experts_grouped_gated_bf16)(h.data, (const int*)ids.data, (const float*)wts.data, gate_up.data,
+                                                                   down.data, meta, (int*)where.data, sorted.data, (float*)z.data, act.data,
+                                                                   (float*)out.data, (float*)y.data, (int)M, (int)W, (int)F, experts, top,
+                                                                   (int)kind, limit, alpha, (hipStream_t)launch_stream());
+    if (rc == 0) {
+      took("[mfma, grouped]");
+      return;
+    }
+    if (rc != 3) check("moe_bf16", rc, "moe_experts_gated(grouped)");
+  }
+  took(rows && top > 1 ? "[rows, sums left]" : "[rows]");
+  Tensor act = ws.tensor("moe.act", h.dtype, {pairs, F});
+  Tensor part = top == 1 ? y : ws.tensor("moe.out", DType::F32, {pairs, W});
+  const bool left = rows && top > 1;
+  int rc = KERNEL("moe", ti_moe_experts_rows_gated)(code(h.dtype, "moe_experts_gated"), h.data, (const int*)ids.data, (const float*)wts.data,
+                                                    gate_up.data, down.data, (float*)z.data, act.data, (float*)part.data,
+                                                    (top == 1 || left) ? nullptr : (float*)y.data, (int)M, (int)W, (int)F, experts, top,
+                                                    (int)kind, limit, alpha, (hipStream_t)launch_stream());
+  check("moe", rc, "moe_experts_gated");
   if (left) {
     rows->t = part;
     rows->gather = nullptr;

@@ -37,6 +37,16 @@
 //   ffn       "moe"         routed experts with sigmoid or softmax scores on the experts' inputs or outputs
 //   block     "post_norm"   x += norm1(mixer(x)); x += norm2(ffn(x)): the sublayers read x itself
 //
+//
+//   norm      "dyt"         Dynamic Tanh: tanh(alpha x) * w + b with one learned number alpha; no mean, no variance
+//   mixer     "attention" with `bias` (biases on q, k, v) and a `pos` beside keys and values of their own sizes
+//   mixer     "latent_attention" a token keeps one normed latent and one rotated key part; keys and values per head come from
+//                           the latent; a learned sink in the softmax's denominator
+//   ffn       "glu"         down(act(gate h, up h)) with act silu(g) u or the clamped g sigmoid(alpha g) (u + 1); optional biases
+//   ffn       "moe" with `activation` "glu_clamped", `score` "softmax_chosen" and a `shared` feed-forward every token takes
+//   block     "keep"        keeps a copy of the residual under a name for a later block of the step
+//   block     "mix_in"      x <- W [x; kept]: the residual and a kept stream through one learned matrix
+//
 // A part gets every size and constant as a parameter and never looks at the model it sits in.
 #include <algorithm>
 #include <cmath>
@@ -524,14 +534,15 @@ class Attention final : public MixerPart {
     qk_norm = p.has("qk_norm") ? p.at("qk_norm").as_bool() : true;
     // capped scores, a query temperature or values of another size than the keys: the kernels that serve these take
     // any sizes up to 256 and neither a per-head norm nor a rotation
-    general = softcap > 0.f || temp_coef != 0.f || v_dim != head_dim || (p.has("general") && p.at("general").as_bool());
+    bias = p.has("bias") && p.at("bias").as_bool();
+    general = softcap > 0.f || temp_coef != 0.f || v_dim != head_dim || bias || (p.has("general") && p.at("general").as_bool());
     if (general) {
       if (head_dim < 1 || head_dim > 256 || v_dim < 1 || v_dim > 256)
         throw ConfigError("attention: key size " + std::to_string(head_dim) + " / value size " + std::to_string(v_dim) +
                           " are not served (up to 256)");
-      if (qk_norm || p.has("pos") || (p.has("shares_kv") && p.at("shares_kv").as_bool()))
-        throw ConfigError("attention: capped scores, a query temperature or a separate value size go with neither a per-head norm, "
-                          "a rotation nor a shared cache");
+      if (qk_norm || (p.has("shares_kv") && p.at("shares_kv").as_bool()))
+        throw ConfigError("attention: capped scores, a query temperature, biases or a separate value size go with neither a per-head norm "
+                          "nor a shared cache");
     } else if (head_dim < 16 || head_dim % 16 || head_dim > 256) {
       // every other attention kernel's range (float32 and bfloat16 alike): refused when the part is built, not at its first step
       throw ConfigError("attention: head_dim " + std::to_string(head_dim) +
@@ -586,9 +597,26 @@ class Attention final : public MixerPart {
       t.emplace_back(join(prefix, "q_norm.weight"), nw);
       if (!shares_kv) t.emplace_back(join(prefix, "k_norm.weight"), nw);
     }
+    if (bias) {
+      // the biases of the projections: the tensor's name with ".b"
+      const std::pair<const std::string*, int64_t> runs[3] = {{&n_q, nq}, {&n_k, nk}, {&n_v, nv}};
+      for (const auto& r : runs) {
+        TensorNeed b;
+        b.shape = {r.second};
+        b.role = TensorNeed::Vector;
+        b.b = 0.3;
+        t.emplace_back(*r.first + ".b", b);
+      }
+    }
     return t;
   }
   void load(WeightSource& src) override {
+    if (bias) {
+      b_qkv = src.alloc(DType::F32, {nq + nk + nv});
+      src.fill(n_q + ".b", b_qkv.rows(0, nq));
+      src.fill(n_k + ".b", b_qkv.rows(nq, nk));
+      src.fill(n_v + ".b", b_qkv.rows(nq + nk, nv));
+    }
     // q, k and v go straight into the fused matrix (the reference builds its fused copy beside the
     // originals and keeps both: /root/reference/src/inference.cu:154-169)
     w_qkv = src.alloc(src.matrix_dtype, {nq + nk + nv, hidden});
@@ -701,7 +729,12 @@ class Attention final : public MixerPart {
     const Tensor pool = ctx.kv_pool(bound.first, bound.second);
     const Ops::CacheView view = ctx.cache_view(bound.first);
     Tensor q = ctx.buf("attn.q", ctx.act_dtype, {M, nq});
-    ctx.ops.qkv_split_write(qkv, ctx.positions, ctx.slots, view, pool, q, heads, kv_heads, head_dim, v_dim, temp_coef, temp_every);
+    Ops::Rotation rot;
+    if (pos && !pos->fused(rot)) throw EngineError("attention: the position encoding '" + std::string(pos->kind_name()) + "' has no fused form");
+    if (bias || pos)
+      ctx.ops.qkv_split_write(qkv, b_qkv, rot, ctx.positions, ctx.slots, view, pool, q, heads, kv_heads, head_dim, v_dim, temp_coef, temp_every);
+    else
+      ctx.ops.qkv_split_write(qkv, ctx.positions, ctx.slots, view, pool, q, heads, kv_heads, head_dim, v_dim, temp_coef, temp_every);
     Tensor a = ctx.buf("attn.out", ctx.act_dtype, {M, no});
     if (v_dim == head_dim)      // the step's tiles through the matrix cores where they serve the size, else row by row
       ctx.ops.attention(work(ctx), ctx.ws, view, q, pool, a, heads, kv_heads, head_dim, scale, window, softcap);
@@ -772,11 +805,12 @@ class Attention final : public MixerPart {
   }
 
   std::vector<std::pair<std::string, Tensor>> held() const override {
-    return {{"w_qkv", w_qkv}, {"w_o", w_o}, {"q_norm_w", q_norm_w}, {"k_norm_w", k_norm_w}};
+    return {{"w_qkv", w_qkv}, {"w_o", w_o}, {"q_norm_w", q_norm_w}, {"k_norm_w", k_norm_w}, {"b_qkv", b_qkv}};
   }
   int64_t hidden = 0, nq = 0, nk = 0, nv = 0, no = 0;
   int heads = 0, kv_heads = 0, head_dim = 0, v_dim = 0, window = 0, temp_every = 0;
-  bool qk_norm = true, shares_kv = false, general = false;
+  bool qk_norm = true, shares_kv = false, general = false, bias = false;
+  Tensor b_qkv;      // `bias`: the biases of q, k and v side by side, 32-bit
   float eps = 1e-6f, scale = 1.f, softcap = 0.f, temp_coef = 0.f;
   std::string n_q, n_k, n_v, n_o;
   std::shared_ptr<PositionPart> pos;
@@ -1504,7 +1538,7 @@ class DiffAttention final : public MixerPart {
 // sum_e expert_e(s_e h); false: its output.  `activation`: "relu2", the square of relu.
 class MoE final : public FeedForwardPart {
  public:
-  MoE(const std::string& prefix, const Json& p) : FeedForwardPart(prefix) {
+  MoE(const std::string& prefix, const Json& p, const PartChildren& children = {}) : FeedForwardPart(prefix) {
     hidden = param_int(p, "hidden");
     intermediate = param_int(p, "intermediate");
     experts = (int)param_int(p, "experts");
@@ -1517,13 +1551,38 @@ class MoE final : public FeedForwardPart {
       throw ConfigError("moe: a width of " + std::to_string(hidden) + " / an expert size of " + std::to_string(intermediate) +
                         " is not served (a row of either must fit 64 KB)");
     const std::string act = p.has("activation") ? p.at("activation").as_string() : "relu2";
-    if (act != "relu2") throw ConfigError("moe: activation '" + act + "' is not served (only 'relu2')");
+    if (act != "relu2" && act != "glu_clamped" && act != "glu_silu")
+      throw ConfigError("moe: activation '" + act + "' is not served (relu2, glu_clamped, glu_silu)");
+    gated = act != "relu2";
+    act_kind = act == "glu_clamped" ? Ops::ClampedGlu : Ops::Silu;
+    if (act == "glu_clamped") {
+      limit = (float)param_float(p, "limit");
+      alpha = p.has("alpha") ? (float)param_float(p, "alpha") : 1.702f;
+      if (!(limit > 0.f)) throw ConfigError("moe: the activation's limit must be positive");
+    }
     const std::string sc = p.has("score") ? p.at("score").as_string() : "sigmoid";
-    if (sc != "sigmoid" && sc != "softmax") throw ConfigError("moe: score '" + sc + "' is not served (sigmoid, softmax)");
-    score = sc == "softmax" ? Ops::Softmax : Ops::Sigmoid;
+    if (sc != "sigmoid" && sc != "softmax" && sc != "softmax_chosen")
+      throw ConfigError("moe: score '" + sc + "' is not served (sigmoid, softmax, softmax_chosen)");
+    score = sc == "softmax" ? Ops::Softmax : sc == "softmax_chosen" ? Ops::SoftmaxChosen : Ops::Sigmoid;
     renormalize = p.has("renormalize") && p.at("renormalize").as_bool();
-    scale_input = !p.has("scale_input") || p.at("scale_input").as_bool();
+    scale_input = gated ? false : (!p.has("scale_input") || p.at("scale_input").as_bool());
+    if (gated && p.has("scale_input") && p.at("scale_input").as_bool()) throw ConfigError("moe: gated experts take their weight on the output");
     n_router = tensor_name(p, "router", prefix, "router");
+    for (const auto& c : children)
+      if (c.first == "shared") shared = std::dynamic_pointer_cast<FeedForwardPart>(c.second);
+    if (!shared && p.has("shared")) {
+      const PartSpec sp = PartSpec::from_json(p.at("shared"));
+      shared = std::dynamic_pointer_cast<FeedForwardPart>(build_part("ffn", sp, join(prefix, sp.name)));
+    }
+    if (shared && !shared->can_store()) throw ConfigError("moe: the shared feed-forward must be able to write its output apart from the residual");
+  }
+  std::vector<std::shared_ptr<Part>> children() const override {
+    if (shared) return {shared};
+    return {};
+  }
+  std::vector<std::string> child_slots() const override {
+    if (shared) return {"shared"};
+    return {};
   }
   const char* kind_name() const override { return "moe"; }
   bool reads_through_ops() const override { return true; }
@@ -1538,6 +1597,7 @@ class MoE final : public FeedForwardPart {
     router.role = TensorNeed::Vector;      // held in 32-bit whatever the engine's dtype
     router.b = 0.1;
     for (int e = 0; e < experts; ++e) {
+      if (gated) t.emplace_back(expert_name(e, "gate"), up);
       t.emplace_back(expert_name(e, "up"), up);
       t.emplace_back(expert_name(e, "down"), down);
     }
@@ -1545,11 +1605,14 @@ class MoE final : public FeedForwardPart {
     return t;
   }
   void load(WeightSource& src) override {
-    // the experts' matrices one under the other: a kernel finds expert e at row e * its rows
-    w_up = src.alloc(src.matrix_dtype, {(int64_t)experts * intermediate, hidden});
+    // the experts' matrices one under the other: a kernel finds expert e at row e * its rows (gated: an expert's gate rows
+    // above its up rows)
+    const int64_t up_rows = gated ? 2 * intermediate : intermediate;
+    w_up = src.alloc(src.matrix_dtype, {(int64_t)experts * up_rows, hidden});
     w_down = src.alloc(src.matrix_dtype, {(int64_t)experts * hidden, intermediate});
     for (int e = 0; e < experts; ++e) {
-      src.fill(expert_name(e, "up"), w_up.rows((int64_t)e * intermediate, intermediate));
+      if (gated) src.fill(expert_name(e, "gate"), w_up.rows((int64_t)e * up_rows, intermediate));
+      src.fill(expert_name(e, "up"), w_up.rows((int64_t)e * up_rows + (gated ? intermediate : 0), intermediate));
       src.fill(expert_name(e, "down"), w_down.rows((int64_t)e * hidden, hidden));
     }
     TensorNeed router;
@@ -1563,11 +1626,25 @@ class MoE final : public FeedForwardPart {
     Tensor ids = ctx.buf("moe.ids", DType::I32, {M, (int64_t)top});
     Tensor wts = ctx.buf("moe.wts", DType::F32, {M, (int64_t)top});
     ctx.ops.moe_route(rows, w_router, ids, wts, top, score, renormalize);
-    ctx.ops.moe_experts(rows, ids, wts, w_up, w_down, y, experts, scale_input, ctx.ws, left);
+    if (gated) ctx.ops.moe_experts_gated(rows, ids, wts, w_up, w_down, y, experts, act_kind, limit, alpha, ctx.ws, left);
+    else ctx.ops.moe_experts(rows, ids, wts, w_up, w_down, y, experts, scale_input, ctx.ws, left);
   }
-  void forward_store(StepContext& ctx, const Rows& h, const Tensor& y) override { run(ctx, h, y, nullptr); }
+  void forward_store(StepContext& ctx, const Rows& h, const Tensor& y) override {
+    run(ctx, h, y, nullptr);
+    if (shared) {      // the expert every token takes, added in 32-bit
+      Tensor ys = ctx.buf("moe.shared", DType::F32, {y.shape[0], hidden});
+      shared->forward_store(ctx, h, ys);
+      ctx.ops.scaled_add(y, ys, Tensor(), Tensor(), Tensor());
+    }
+  }
   // the sum over a token's experts may be left to the norm that reads the result
   void forward_rows(StepContext& ctx, const Rows& h, const Tensor& y, Ops::GatheredRows& rows) override {
+    if (shared) {
+      forward_store(ctx, h, y);
+      rows = Ops::GatheredRows();
+      rows.t = y;
+      return;
+    }
     run(ctx, h, y, &rows);
     if (!rows.t.defined()) rows.t = y;
   }
@@ -1581,8 +1658,295 @@ class MoE final : public FeedForwardPart {
   int experts = 0, top = 0;
   Ops::RouterScore score = Ops::Sigmoid;
   bool renormalize = false, scale_input = true;
+  bool gated = false;                      // `activation` glu_*: experts hold gate, up and down; the weight is on the output
+  Ops::GatedAct act_kind = Ops::Silu;
+  float limit = 0.f, alpha = 1.702f;       // glu_clamped: g = min(g, limit), u = clamp(u, -limit, limit), g sigmoid(alpha g) (u + 1)
+  std::shared_ptr<FeedForwardPart> shared; // `shared`: a feed-forward every token takes, added to the experts' sum
   std::string n_router;
   Tensor w_up, w_down, w_router;
+};
+
+// Dynamic Tanh in the place of a norm: y = tanh(alpha x) * w + b, alpha one learned number, w and b vectors; no mean and no
+// variance is taken.  Tensor names: `tensor` (default prefix + ".weight"), and that name with ".alpha" and ".b".
+class DynamicTanh final : public NormPart {
+ public:
+  DynamicTanh(const std::string& prefix, const Json& p) : NormPart(prefix) {
+    dim = param_int(p, "dim");
+    name = tensor_name(p, "tensor", prefix, "weight");
+    if (dim <= 0) throw ConfigError("dyt: dim must be positive");
+  }
+  const char* kind_name() const override { return "dyt"; }
+  bool reads_through_ops() const override { return true; }
+  std::vector<std::pair<std::string, TensorNeed>> tensors() const override {
+    TensorNeed w, a, b;
+    w.shape = b.shape = {dim};
+    w.role = a.role = b.role = TensorNeed::Vector;
+    w.a = 1.0;
+    w.b = 0.1;
+    a.a = 0.5;
+    a.b = 0.05;
+    b.b = 0.1;
+    return {{name, w}, {name + ".alpha", a}, {name + ".b", b}};
+  }
+  void load(WeightSource& src) override {
+    const auto t = tensors();
+    weight = src.fetch(t[0].first, t[0].second);
+    alpha = src.fetch(t[1].first, t[1].second);
+    bias = src.fetch(t[2].first, t[2].second);
+  }
+  Rows forward(StepContext& ctx, const Tensor& x, const int* rows, int64_t n_rows, bool) override {
+    const int64_t n = rows ? n_rows : x.shape[0];
+    Rows r;
+    r.t = ctx.buf("norm.out", ctx.act_dtype, {n, dim});
+    ctx.ops.dyt(x, alpha, weight, bias, r.t, rows, n_rows);
+    return r;
+  }
+  std::vector<std::pair<std::string, Tensor>> held() const override { return {{"weight", weight}, {"alpha", alpha}, {"bias", bias}}; }
+  int64_t dim = 0;
+  std::string name;
+  Tensor weight, alpha, bias;
+};
+
+// A gated feed-forward: down(act(gate h, up h)).  `activation` "silu": silu(g) u; "clamped" (`limit`, `alpha` default 1.702):
+// g = min(g, limit), u = clamp(u, -limit, limit), g sigmoid(alpha g) (u + 1).  `bias`: every projection has a bias (the
+// tensor's name with ".b").  The first product leaves 32-bit sums of [gate | up] (one stacked weight), the activation is
+// taken in 32-bit and rounded once.  Tensor names: prefix + ".gate", ".up", ".down" unless the parameters give them.
+class GatedFFN final : public FeedForwardPart {
+ public:
+  GatedFFN(const std::string& prefix, const Json& p) : FeedForwardPart(prefix) {
+    hidden = param_int(p, "hidden");
+    intermediate = param_int(p, "intermediate");
+    if (hidden <= 0 || intermediate <= 0) throw ConfigError("glu feed-forward: sizes must be positive");
+    const std::string act = p.has("activation") ? p.at("activation").as_string() : "silu";
+    if (act != "silu" && act != "clamped") throw ConfigError("glu feed-forward: activation '" + act + "' is not served (silu, clamped)");
+    kind = act == "clamped" ? Ops::ClampedGlu : Ops::Silu;
+    if (kind == Ops::ClampedGlu) {
+      limit = (float)param_float(p, "limit");
+      alpha = p.has("alpha") ? (float)param_float(p, "alpha") : 1.702f;
+      if (!(limit > 0.f)) throw ConfigError("glu feed-forward: limit must be positive");
+    }
+    bias = p.has("bias") && p.at("bias").as_bool();
+    n_gate = tensor_name(p, "gate", prefix, "gate");
+    n_up = tensor_name(p, "up", prefix, "up");
+    n_down = tensor_name(p, "down", prefix, "down");
+  }
+  const char* kind_name() const override { return "glu"; }
+  bool reads_through_ops() const override { return true; }
+  bool can_store() const override { return true; }
+  std::vector<std::pair<std::string, TensorNeed>> tensors() const override {
+    TensorNeed up, down, bu, bd;
+    up.shape = {intermediate, hidden};
+    down.shape = {hidden, intermediate};
+    bu.shape = {intermediate};
+    bd.shape = {hidden};
+    bu.role = bd.role = TensorNeed::Vector;
+    bu.b = bd.b = 0.2;
+    std::vector<std::pair<std::string, TensorNeed>> t = {{n_gate, up}, {n_up, up}, {n_down, down}};
+    if (bias) {
+      t.emplace_back(n_gate + ".b", bu);
+      t.emplace_back(n_up + ".b", bu);
+      t.emplace_back(n_down + ".b", bd);
+    }
+    return t;
+  }
+  void load(WeightSource& src) override {
+    w_gate_up = src.alloc(src.matrix_dtype, {2 * intermediate, hidden});
+    src.fill(n_gate, w_gate_up.rows(0, intermediate));
+    src.fill(n_up, w_gate_up.rows(intermediate, intermediate));
+    TensorNeed down;
+    down.shape = {hidden, intermediate};
+    w_down = src.fetch(n_down, down);
+    if (bias) {
+      b_gate_up = src.alloc(DType::F32, {2 * intermediate});
+      src.fill(n_gate + ".b", b_gate_up.rows(0, intermediate));
+      src.fill(n_up + ".b", b_gate_up.rows(intermediate, intermediate));
+      TensorNeed bd;
+      bd.shape = {hidden};
+      bd.role = TensorNeed::Vector;
+      b_down = src.fetch(n_down + ".b", bd);
+    }
+  }
+  void run(StepContext& ctx, const Rows& h, const Tensor& out, Ops::Epilogue epi) {
+    const int64_t M = h.t.shape[0];
+    Tensor z = ctx.buf("glu.z", DType::F32, {M, 2 * intermediate});
+    ctx.ops.linear(h, w_gate_up, z, Ops::Store);
+    Tensor y = ctx.buf("glu.y", ctx.act_dtype, {M, intermediate});
+    ctx.ops.gated_act(z, b_gate_up, y, kind, limit, alpha);
+    ctx.ops.linear(y, w_down, out, epi, false);
+    if (bias) ctx.ops.add_row(out, b_down);
+  }
+  void forward(StepContext& ctx, const Rows& h, const Tensor& x) override { run(ctx, h, x, Ops::Add); }
+  void forward_store(StepContext& ctx, const Rows& h, const Tensor& y) override { run(ctx, h, y, Ops::Store); }
+  std::vector<std::pair<std::string, Tensor>> held() const override {
+    return {{"w_gate_up", w_gate_up}, {"w_down", w_down}, {"b_gate_up", b_gate_up}, {"b_down", b_down}};
+  }
+  int64_t hidden = 0, intermediate = 0;
+  Ops::GatedAct kind = Ops::Silu;
+  float limit = 0.f, alpha = 1.702f;
+  bool bias = false;
+  std::string n_gate, n_up, n_down;
+  Tensor w_gate_up, w_down, b_gate_up, b_down;
+};
+
+// Latent attention.  Per token the mixer keeps a latent c of `kv_rank` numbers and one rotated key part of `rot_dim` numbers
+// that all heads share (paged rows [kv_rank + rot_dim]); keys and values are never kept per head.  q = W_q h, head by head
+// [head_dim unrotated | rot_dim rotated]; W_dkv h has kv_rank + rot_dim rows: the first kv_rank, divided by their root mean
+// square (eps) and multiplied by the vector `dkv.norm`, are c, the rest is the key part, rotated by the child `pos` as every
+// head's last rot_dim query entries are.  A head's unrotated key is W_uk c (head_dim rows a head), its value W_uv c
+// (v_head_dim rows a head); score = (q_plain . k_plain + q_rot . k_rot) scale; causal (`window` optional); the softmax's
+// denominator also holds exp(sink_h), a learned number a head (`sink`, optional).  Then the output projection.
+// Scores, softmax, the latent's norm and the rotation are 32-bit.  Tensor names: prefix + ".q", ".dkv", ".dkv.norm", ".uk",
+// ".uv", ".sink", ".o".
+class LatentAttention final : public MixerPart {
+ public:
+  LatentAttention(const std::string& prefix, const Json& p, const PartChildren& children) : MixerPart(prefix) {
+    hidden = param_int(p, "hidden");
+    heads = (int)param_int(p, "heads");
+    dim = (int)param_int(p, "head_dim");
+    rot_dim = (int)param_int(p, "rot_dim");
+    v_dim = p.has("v_head_dim") ? (int)param_int(p, "v_head_dim") : dim;
+    rank = (int)param_int(p, "kv_rank");
+    if (heads <= 0 || dim < 0 || rot_dim < 0 || dim + rot_dim <= 0 || v_dim <= 0 || rank <= 0)
+      throw ConfigError("latent_attention: sizes must be positive");
+    if (rank + rot_dim > 768 || dim > 1536)
+      throw ConfigError("latent_attention: a latent of " + std::to_string(rank) + " + " + std::to_string(rot_dim) + " is not served (up to 768 together)");
+    eps = (float)(p.has("eps") ? param_float(p, "eps") : 1e-6);
+    scale = p.has("scale") ? (float)param_float(p, "scale") : (float)(1.0 / std::sqrt((double)(dim + rot_dim)));
+    window = p.has("window") ? (int)param_int(p, "window") : 0;
+    has_sink = !p.has("sink") || p.at("sink").as_bool();
+    for (const auto& c : children)
+      if (c.first == "pos") pos = std::dynamic_pointer_cast<PositionPart>(c.second);
+    if (!pos && p.has("pos")) pos = std::dynamic_pointer_cast<PositionPart>(build_part("pos", PartSpec::from_json(p.at("pos")), prefix));
+    nq = (int64_t)heads * (dim + rot_dim);
+    nkv = (int64_t)rank + rot_dim;
+  }
+  const char* kind_name() const override { return "latent_attention"; }
+  bool can_store() const override { return true; }
+  bool takes_lazy_norm() const override { return true; }
+  bool reads_through_ops() const override { return true; }
+  std::vector<std::shared_ptr<Part>> children() const override {
+    if (pos) return {pos};
+    return {};
+  }
+  std::vector<std::string> child_slots() const override {
+    if (pos) return {"pos"};
+    return {};
+  }
+  std::string name(const char* t) const { return join(prefix, t); }
+  std::vector<std::pair<std::string, TensorNeed>> tensors() const override {
+    TensorNeed q, dkv, nw, uk, uv, sk, o;
+    q.shape = {nq, hidden};
+    dkv.shape = {nkv, hidden};
+    nw.shape = {(int64_t)rank};
+    nw.role = TensorNeed::Vector;
+    nw.a = 1.0;
+    nw.b = 0.1;
+    uk.shape = {(int64_t)heads * dim, (int64_t)rank};
+    uv.shape = {(int64_t)heads * v_dim, (int64_t)rank};
+    sk.shape = {(int64_t)heads};
+    sk.role = TensorNeed::Vector;
+    sk.b = 1.0;
+    o.shape = {hidden, (int64_t)heads * v_dim};
+    std::vector<std::pair<std::string, TensorNeed>> t = {{name("q"), q}, {name("dkv"), dkv}, {name("dkv.norm"), nw}, {name("uk"), uk},
+                                                         {name("uv"), uv}};
+    if (has_sink) t.emplace_back(name("sink"), sk);
+    t.emplace_back(name("o"), o);
+    return t;
+  }
+  void load(WeightSource& src) override {
+    const auto t = tensors();
+    w_in = src.alloc(src.matrix_dtype, {nq + nkv, hidden});      // queries above the down-projection: one product
+    src.fill(name("q"), w_in.rows(0, nq));
+    src.fill(name("dkv"), w_in.rows(nq, nkv));
+    for (const auto& kv : t) {
+      if (kv.first == name("dkv.norm")) norm_w = src.fetch(kv.first, kv.second);
+      if (kv.first == name("uk")) w_uk = src.fetch(kv.first, kv.second);
+      if (kv.first == name("uv")) w_uv = src.fetch(kv.first, kv.second);
+      if (kv.first == name("sink")) sink = src.fetch(kv.first, kv.second);
+      if (kv.first == name("o")) w_o = src.fetch(kv.first, kv.second);
+    }
+  }
+  bool has_cache() const override { return true; }
+  CacheNeed cache_need() const override {
+    CacheNeed n;
+    n.kind = CacheNeed::PagedRows;
+    n.row_shape = {nkv};
+    n.window = window;
+    return n;
+  }
+  void run(StepContext& ctx, const Rows& h, const Tensor& out, Ops::Epilogue epi) {
+    const int64_t M = h.t.shape[0];
+    Tensor proj = ctx.buf("latent.proj", DType::F32, {M, nq + nkv});
+    ctx.ops.linear(h, w_in, proj, Ops::Store);
+    const auto bound = ctx.binding(this);
+    const Tensor pool = ctx.kv_pool(bound.first, bound.second);
+    const Ops::CacheView view = ctx.cache_view(bound.first);
+    Ops::Rotation rot;
+    if (pos && !pos->fused(rot)) throw EngineError("latent_attention: the position encoding '" + std::string(pos->kind_name()) + "' has no fused form");
+    ctx.ops.latent_prep(proj, (int)nq, norm_w, eps, rot, ctx.positions, ctx.slots, view, pool, heads, dim, rot_dim, rank);
+    Tensor a = ctx.buf("latent.out", ctx.act_dtype, {M, (int64_t)heads * v_dim});
+    ctx.ops.latent_attention(proj, w_uk, w_uv, sink, pool, view, ctx.positions, ctx.slots, a, heads, dim, rot_dim, rank, v_dim, scale,
+                             window, ctx.ws);
+    ctx.ops.linear(a, w_o, out, epi, false);
+  }
+  void forward(StepContext& ctx, const Rows& h, const Tensor& x) override { run(ctx, h, x, Ops::Add); }
+  void forward_store(StepContext& ctx, const Rows& h, const Tensor& y) override { run(ctx, h, y, Ops::Store); }
+  std::vector<std::pair<std::string, Tensor>> held() const override {
+    return {{"w_in", w_in}, {"norm_w", norm_w}, {"w_uk", w_uk}, {"w_uv", w_uv}, {"sink", sink}, {"w_o", w_o}};
+  }
+  int64_t hidden = 0, nq = 0, nkv = 0;
+  int heads = 0, dim = 0, rot_dim = 0, v_dim = 0, rank = 0, window = 0;
+  bool has_sink = true;
+  float eps = 1e-6f, scale = 1.f;
+  std::shared_ptr<PositionPart> pos;
+  Tensor w_in, norm_w, w_uk, w_uv, sink, w_o;
+};
+
+// Keeps a copy of the residual as it stands, under `name`, for a later block of the same step (the embedding's output that
+// a looped run of layers mixes in again before each pass).
+class KeepBlock final : public BlockPart {
+ public:
+  KeepBlock(const std::string& prefix, const Json& p) : BlockPart(prefix) {
+    name = p.has("name") ? p.at("name").as_string() : std::string("kept");
+  }
+  const char* kind_name() const override { return "keep"; }
+  void forward(StepContext& ctx, const Tensor& x) override {
+    ctx.ops.flush();
+    Tensor k = ctx.buf("kept." + name, DType::F32, {x.shape[0], x.shape[1]});
+    ctx.ops.fill_zero(k.data, k.bytes());
+    ctx.ops.scaled_add(k, x, Tensor(), Tensor(), Tensor());
+  }
+  std::string name;
+};
+
+// x <- W [x; kept]: the residual and the stream a `keep` block left under `from`, side by side through one learned matrix
+// [dim, 2 dim] (the residual's columns first).  `tensor`: the matrix's name; several such blocks share it.
+class MixInBlock final : public BlockPart {
+ public:
+  MixInBlock(const std::string& prefix, const Json& p) : BlockPart(prefix) {
+    dim = param_int(p, "dim");
+    from = p.has("from") ? p.at("from").as_string() : std::string("kept");
+    name = tensor_name(p, "tensor", prefix, "weight");
+  }
+  const char* kind_name() const override { return "mix_in"; }
+  std::vector<std::pair<std::string, TensorNeed>> tensors() const override {
+    TensorNeed n;
+    n.shape = {dim, 2 * dim};
+    return {{name, n}};
+  }
+  void load(WeightSource& src) override { w = src.fetch(name, tensors()[0].second); }
+  void forward(StepContext& ctx, const Tensor& x) override {
+    ctx.ops.flush();
+    const int64_t M = x.shape[0];
+    const Tensor kept = ctx.buf("kept." + from, DType::F32, {M, dim});
+    Tensor both = ctx.buf("mix_in.rows", ctx.act_dtype, {M, 2 * dim});
+    ctx.ops.concat_round(x, kept, both);
+    ctx.ops.linear(both, w, x, Ops::Store);
+  }
+  std::vector<std::pair<std::string, Tensor>> held() const override { return {{"w", w}}; }
+  int64_t dim = 0;
+  std::string from, name;
+  Tensor w;
 };
 
 // x += norm1(mixer(x)); x += norm2(ffn(x)).  The sublayers read the residual itself (rounded to the compute dtype where
@@ -1668,9 +2032,22 @@ void register_builtin_parts() {
   register_part("mixer", "diff_attention", [](const std::string& prefix, const Json& p, const PartChildren& c) {
     return std::make_shared<DiffAttention>(prefix, p, c);
   });
-  register_part("ffn", "moe", [](const std::string& prefix, const Json& p, const PartChildren&) {
-    return std::make_shared<MoE>(prefix, p);
+  register_part("ffn", "moe", [](const std::string& prefix, const Json& p, const PartChildren& c) {
+    return std::make_shared<MoE>(prefix, p, c);
   });
+  register_part("norm", "dyt", [](const std::string& prefix, const Json& p, const PartChildren&) {
+    return std::make_shared<DynamicTanh>(prefix, p);
+  });
+  register_part("ffn", "glu", [](const std::string& prefix, const Json& p, const PartChildren&) {
+    return std::make_shared<GatedFFN>(prefix, p);
+  });
+  register_part("mixer", "latent_attention", [](const std::string& prefix, const Json& p, const PartChildren& c) {
+    return std::make_shared<LatentAttention>(prefix, p, c);
+  });
+  register_part("block", "keep",
+                [](const std::string& prefix, const Json& p, const PartChildren&) { return std::make_shared<KeepBlock>(prefix, p); });
+  register_part("block", "mix_in",
+                [](const std::string& prefix, const Json& p, const PartChildren&) { return std::make_shared<MixInBlock>(prefix, p); });
   register_part("block", "post_norm",
                 [](const std::string& prefix, const Json&, const PartChildren& c) { return std::make_shared<PostNormBlock>(prefix, c); },
                 {{"norm1", "norm"}, {"mixer", "mixer"}, {"norm2", "norm?"}, {"ffn", "ffn?"}});
