@@ -1239,6 +1239,37 @@ int ti_ops_call(void* ops_, const char* op_, const ti_tensor* t, int n_t, const 
     // qkv, positions, slots, table, pool [pages, kv_heads, P, dk + dv], q_out; heads, kv_heads, dk, dv, coef, every
     ops.qkv_split_write(arg(0), iptr(1), iptr(2), view_of(3, arg(4)), arg(4), arg(5), (int)num(0), (int)num(1), (int)num(2),
                         (int)num(3), (float)num(4), (int)num(5));
+  } else if (op == "qkv_prep_write") {
+    // qkv, bias, inv_freq, rope_table, positions, slots, table, pool, q_out; heads, kv_heads, dk, dv, coef, every, rotated entries, mag
+    Ops::Rotation r = rotation(2, 3);
+    r.dims = (int)num(6);
+    r.mag = (float)num(7);
+    ops.qkv_split_write(arg(0), arg(1), r, iptr(4), iptr(5), view_of(6, arg(7)), arg(7), arg(8), (int)num(0), (int)num(1), (int)num(2),
+                        (int)num(3), (float)num(4), (int)num(5));
+  } else if (op == "dyt") {
+    // x, alpha, w, b (may be absent), out, rows (may be absent)
+    const bool rows = n_t > 5 && arg(5).defined();
+    ops.dyt(arg(0), arg(1), arg(2), arg(3), arg(4), rows ? iptr(5) : nullptr, rows ? arg(5).shape[0] : 0);
+  } else if (op == "gated_act") {
+    // z, bias (may be absent), out; kind, limit, alpha
+    ops.gated_act(arg(0), arg(1), arg(2), (Ops::GatedAct)(int)num(0), (float)num(1), (float)num(2));
+  } else if (op == "concat_round") {
+    ops.concat_round(arg(0), arg(1), arg(2));
+  } else if (op == "latent_prep") {
+    // proj, norm_w, inv_freq, rope_table, positions, slots, table, pool; off_kv, eps, heads, dim, rot_dim, rank, rotated entries, mag
+    Ops::Rotation r = rotation(2, 3);
+    r.dims = (int)num(6);
+    r.mag = (float)num(7);
+    ops.latent_prep(arg(0), (int)num(0), arg(1), (float)num(1), r, iptr(4), iptr(5), view_of(6, arg(7)), arg(7), (int)num(2), (int)num(3),
+                    (int)num(4), (int)num(5));
+  } else if (op == "latent_attention") {
+    // proj, w_uk, w_uv, sink (may be absent), pool, table, positions, slots, out; heads, dim, rot_dim, rank, v_dim, scale, window
+    ops.latent_attention(arg(0), arg(1), arg(2), arg(3), arg(4), view_of(5, arg(4)), iptr(6), iptr(7), arg(8), (int)num(0), (int)num(1),
+                         (int)num(2), (int)num(3), (int)num(4), (float)num(5), (int)num(6), workspace_of(&ops));
+  } else if (op == "moe_experts_gated") {
+    // h, ids, wts, gate_up, down, y; experts, kind, limit, alpha
+    ops.moe_experts_gated(arg(0), arg(1), arg(2), arg(3), arg(4), arg(5), (int)num(0), (Ops::GatedAct)(int)num(1), (float)num(2),
+                          (float)num(3), workspace_of(&ops));
   } else if (op == "attention_capped") {
     // q, pool, table, positions, slots, out; heads, kv_heads, dk, dv, scale, softcap, window
     ops.attention_capped(arg(0), arg(1), view_of(2, arg(1)), iptr(3), iptr(4), arg(5), (int)num(0), (int)num(1), (int)num(2),

@@ -98,7 +98,9 @@ _LIB_OF = {"embed": "core", "rmsnorm": "core", "rope_neox": "core", "rope_table"
            "scaled_add": "pointwise", "qkv_split_write": "pointwise", "attention_capped": "attention_generic",
            "mlstm_scan": "recurrent", "gated_head_norm": "recurrent", "norm_residual": "residual", "round_rows": "residual",
            "scale": "residual", "short_conv": "diff_attention", "diff_qk_prep": "diff_attention", "diff_attention": "diff_attention",
-           "moe_route": "moe", "moe_experts": "moe"}
+           "moe_route": "moe", "moe_experts": "moe", "moe_experts_gated": "moe", "qkv_prep_write": "pointwise", "dyt": "pointwise",
+           "gated_act": "pointwise", "concat_round": "pointwise", "latent_prep": "latent_attention",
+           "latent_attention": "latent_attention"}
 
 
 class Ops:
@@ -398,7 +400,43 @@ class Ops:
         self._call("diff_attention", tensors, numbers, libs=libs)
 
     def moe_route(self, h, router, ids, wts, top, score="sigmoid", renormalize=False):
-        self._call("moe_route", [h, router, ids, wts], [top, {"sigmoid": 0, "softmax": 1}[score], int(bool(renormalize))])
+        """score "softmax_chosen": the largest logits are chosen and the weights are the softmax over the chosen logits alone."""
+        self._call("moe_route", [h, router, ids, wts], [top, {"sigmoid": 0, "softmax": 1, "softmax_chosen": 2}[score], int(bool(renormalize))])
+
+    def moe_experts_gated(self, h, ids, wts, gate_up, down, y, experts, activation="clamped", limit=0.0, alpha=1.702):
+        """y f32 [M, W] = sum_k s_k down_e act(gate_e h, up_e h); gate_up [experts 2F, W] holds an expert's gate rows above its up rows."""
+        libs = ["moe"] + (["moe_bf16"] if h.dtype == native.torch().bfloat16 else [])
+        self._call("moe_experts_gated", [h, ids, wts, gate_up, down, y], [experts, {"silu": 0, "clamped": 1}[activation], limit, alpha], libs=libs)
+
+    # ---- Dynamic Tanh, gated activations, biased and partly rotated q/k/v, latent attention
+    def dyt(self, x, alpha, w, b, out, rows=None):
+        """out[r] = tanh(alpha x[rows[r] or r]) * w + b; x float32, alpha float32 [1]."""
+        self._call("dyt", [x, alpha, w, b, out, rows])
+
+    def gated_act(self, z, bias, out, activation="silu", limit=0.0, alpha=1.702):
+        """z f32 [R, 2F] = [gate | up] (+ bias [2F]); "silu": silu(g) u; "clamped": g = min(g, limit), u = clamp(u, +-limit),
+        g sigmoid(alpha g) (u + 1)."""
+        self._call("gated_act", [z, bias, out], [{"silu": 0, "clamped": 1}[activation], limit, alpha])
+
+    def concat_round(self, a, b, out):
+        self._call("concat_round", [a, b, out])
+
+    def qkv_prep_write(self, qkv, bias, inv_freq, rope_table, positions, slots, table, pool, q_out, heads, kv_heads, dk, dv,
+                       rot_dims=0, mag=1.0, coef=0.0, every=1):
+        """`qkv_split_write` with a bias on every column first and the rotation of the first rot_dims entries of every query and key head."""
+        self._call("qkv_prep_write", [qkv, bias, inv_freq, rope_table, positions, slots, table, pool, q_out],
+                   [heads, kv_heads, dk, dv, coef, every, rot_dims, mag])
+
+    def latent_prep(self, proj, norm_w, inv_freq, rope_table, positions, slots, table, pool, off_kv, eps, heads, dim, rot_dim, rank,
+                    rot_dims=0, mag=1.0):
+        """proj f32 [M, >= off_kv + rank + rot_dim]: the latent normed and the shared key part rotated into pool [pages, P, rank + rot_dim];
+        the heads' rotated query parts turned in place."""
+        self._call("latent_prep", [proj, norm_w, inv_freq, rope_table, positions, slots, table, pool],
+                   [off_kv, eps, heads, dim, rot_dim, rank, rot_dims, mag])
+
+    def latent_attention(self, proj, w_uk, w_uv, sink, pool, table, positions, slots, out, heads, dim, rot_dim, rank, v_dim, scale, window=0):
+        self._call("latent_attention", [proj, w_uk, w_uv, sink, pool, table, positions, slots, out],
+                   [heads, dim, rot_dim, rank, v_dim, scale, int(window or 0)])
 
     def moe_experts(self, h, ids, wts, up, down, y, experts, scale_input=True):
         """y f32 [M, W] = sum over a token's experts; up [experts F, W], down [experts W, F]."""
