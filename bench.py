@@ -34,6 +34,15 @@ size each over values of the full head size (the projections have the sizes of t
 model's own), a short convolution of four taps, keys visible inside blocks of
 `--mask-size` positions, and `--experts` experts of which a token takes `--top`, each
 sized so that a token's experts do the arithmetic of the model's dense feed-forward.
+
+`--design nazorax` does the same for a Nazorax decoder: parallel layers behind a Dynamic
+Tanh, as mixers `--mixers attention` (biased, rotated attention with the model's heads
+under a window of `--window` positions), `latent` (latent attention with the model's
+heads: 128 unrotated and 64 rotated entries a head, a latent of 512, a sink) or
+`alternate`; as feed-forward `--ffn dense` (SwiGLU with biases at the model's width) or
+`moe` (`--experts` clamped experts of which a token takes `--top`, plus a shared one,
+sized so that a token's experts and the shared one together do the dense feed-forward's
+arithmetic); the embedding's output is mixed in once in front of the layers.
 """
 from __future__ import annotations
 
@@ -89,6 +98,23 @@ def mumasun_config(base, experts, top, mask_size):
                  mlp=dict(kind="moe", expert=dict(ff=ff), router=dict(experts=experts, top=top)))
     return dict(architecture="Mumasun", width=H, vocab=base["vocab_size"], logit_scale=1.0, norm=dict(eps=1e-6),
                 layers=[layer] * base["num_hidden_layers"])
+
+
+def nazorax_config(base, mixers, ffn, experts, top, window):
+    """A Nazorax config.json with the layer widths of the Qwen3 configuration `base`."""
+    H, F, hd = base["hidden_size"], base["intermediate_size"], base["head_dim"]
+    ff = max(64, (F // (top + 1)) // 64 * 64)            # top experts and the shared one do what the dense one of F does
+    mlp = dict(kind="dense", ff=F) if ffn == "dense" else dict(kind="moe", expert=dict(ff=ff, limit=7.0), router=dict(experts=experts, top=top),
+                                                               shared=dict(ff=ff, limit=7.0))
+    attention = dict(type="attention", mixer=dict(heads=base["num_attention_heads"], kv_heads=base["num_key_value_heads"], dim=hd, vdim=hd,
+                                                  scale=hd ** -0.5, mask=dict(size=window), rot=dict(base=1000000.0, dims=hd)), mlp=mlp)
+    latent = dict(type="latent_attention",
+                  mixer=dict(heads=base["num_attention_heads"], dim=hd, rot_dim=hd // 2, vdim=hd, kv_rank=4 * hd, scale=(hd + hd // 2) ** -0.5,
+                             rot=dict(base=1000000.0, dims=hd // 2, scaling=dict(factor=4.0, original=8192, fast=32.0, slow=1.0))), mlp=mlp)
+    kinds = {"attention": [attention], "latent": [latent], "alternate": [attention, latent]}[mixers]
+    L = base["num_hidden_layers"]
+    return dict(architecture="Nazorax", width=H, vocab=base["vocab_size"], norm=dict(eps=1e-6), loop=dict(start=0, stop=L, times=1),
+                layers=[kinds[i % len(kinds)] for i in range(L)])
 
 
 MAX_SEQ = 4096            # context length a request may reach (more if --context asks for it)
@@ -406,13 +432,15 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--model", choices=sorted(MODELS), default="0.6b", help="whose layer sizes the model has")
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
-    ap.add_argument("--design", choices=["qwen3", "miterax", "mumasun"], default="qwen3",
-                    help="miterax / mumasun: a decoder of that design with the layer widths of --model instead (see --mixers; --experts, --top, --mask-size)")
-    ap.add_argument("--experts", type=int, default=8, help="--design mumasun: experts per layer")
-    ap.add_argument("--top", type=int, default=2, help="--design mumasun: experts a token takes")
+    ap.add_argument("--design", choices=["qwen3", "miterax", "mumasun", "nazorax"], default="qwen3",
+                    help="miterax / mumasun / nazorax: a decoder of that design with the layer widths of --model instead (see --mixers; --experts, --top, --mask-size; --ffn, --window)")
+    ap.add_argument("--experts", type=int, default=8, help="--design mumasun / nazorax: experts per layer")
+    ap.add_argument("--top", type=int, default=2, help="--design mumasun / nazorax: experts a token takes")
+    ap.add_argument("--ffn", choices=["dense", "moe"], default="moe", help="--design nazorax: the feed-forward of its layers")
+    ap.add_argument("--window", type=int, default=1024, help="--design nazorax: positions an attention layer's window keeps")
     ap.add_argument("--mask-size", type=int, default=4096, help="--design mumasun: positions of a block of visible keys")
-    ap.add_argument("--mixers", choices=["attention", "mlstm", "alternate"], default="alternate",
-                    help="--design miterax: the mixer of its layers")
+    ap.add_argument("--mixers", choices=["attention", "mlstm", "latent", "alternate"], default="alternate",
+                    help="--design miterax (attention, mlstm, alternate) / nazorax (attention, latent, alternate): the mixer of its layers")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=2048, help="cached tokens each decoding request holds")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
@@ -449,6 +477,14 @@ def main() -> int:
     if args.design == "mumasun":
         cfg = mumasun_config(cfg, args.experts, args.top, args.mask_size)
         model_name = f"Mumasun ({args.top} of {args.experts} experts, blocks of {args.mask_size}) at {NAMES[args.model]} sizes"
+    if args.design == "nazorax":
+        if args.mixers == "mlstm":
+            ap.error("--design nazorax has the mixers attention, latent and alternate")
+        cfg = nazorax_config(cfg, args.mixers, args.ffn, args.experts, args.top, args.window)
+        what = "dense feed-forward" if args.ffn == "dense" else f"{args.top} of {args.experts} experts and a shared one"
+        model_name = f"Nazorax ({args.mixers} mixers, {what}) at {NAMES[args.model]} sizes"
+    elif args.mixers == "latent":
+        ap.error("--mixers latent goes with --design nazorax")
     rng = np.random.default_rng(0)
     context, prefill_tokens = args.context, args.prefill_tokens
     max_seq = max(MAX_SEQ, context + args.warmup + args.steps + 64, prefill_tokens, args.cached + args.portion)

@@ -128,8 +128,7 @@ Json nazorax_typed_config(const Json& d) {
       }
       mo.set("rot", read_rot(m, mw, dim));
     } else if (type.as_string() == "latent_attention") {
-      const int64_t dim = need_int(m, "dim", mw, 0), rot_dim = need_int(m, "rot_dim", mw, 0);
-      if (dim + rot_dim < 1) throw ConfigError("config.json: " + mw + "'dim' + 'rot_dim' must be at least 1");
+      const int64_t dim = need_int(m, "dim", mw), rot_dim = need_int(m, "rot_dim", mw, 0);
       mo.set("dim", dim);
       mo.set("rot_dim", rot_dim);
       mo.set("vdim", given(m, "vdim") ? need_int(m, "vdim", mw) : dim);

@@ -736,7 +736,7 @@ class Attention final : public MixerPart {
     else
       ctx.ops.qkv_split_write(qkv, ctx.positions, ctx.slots, view, pool, q, heads, kv_heads, head_dim, v_dim, temp_coef, temp_every);
     Tensor a = ctx.buf("attn.out", ctx.act_dtype, {M, no});
-    if (v_dim == head_dim)      // the step's tiles through the matrix cores where they serve the size, else row by row
+    if (v_dim == head_dim && head_dim % 16 == 0)      // the step's tiles through the matrix cores where they serve the size, else row by row
       ctx.ops.attention(work(ctx), ctx.ws, view, q, pool, a, heads, kv_heads, head_dim, scale, window, softcap);
     else
       ctx.ops.attention_capped(q, pool, view, ctx.positions, ctx.slots, a, heads, kv_heads, head_dim, v_dim, scale, softcap, window);
