@@ -242,6 +242,79 @@ def test_latent_attention_with_a_sink(ops, dtype, H, d, r, dv, R, P, scaling):
         assert err.max() < bound * max(1.0, np.abs(want).max()), (i, err.max())
 
 
+@pytest.mark.parametrize("H,d,r,dv,R,P,window", [(4, 32, 16, 32, 64, 16, 0), (8, 64, 32, 64, 128, 16, 0), (16, 128, 64, 128, 512, 16, 0),
+                                                  (3, 8, 8, 16, 16, 32, 0), (20, 24, 8, 48, 96, 16, 0), (2, 40, 24, 16, 240, 64, 0),
+                                                  (4, 32, 32, 48, 128, 16, 50)])
+def test_latent_attention_on_the_matrix_cores(ops, H, d, r, dv, R, P, window):
+    """bfloat16, pages that hold the latents transposed as well: the request as one portion in tiles of 64 rows (the last one
+    short), every row as a single token, some rows as tiles beside others as single tokens, and single tokens with their keys
+    split over several workgroups, against the plain mixer; the row-wise kernels read the same pages."""
+    rng = np.random.default_rng(H * 100 + R)
+    T, W, eps = (150 if R < 512 else 100), 48, 1e-5
+    m = dict(heads=H, dim=d, rot_dim=r, vdim=dv, kv_rank=R, scale=1.2 / math.sqrt(d + r),
+             rot=dict(base=500.0, dims=r, scaling=nm.yarn(4.0, 32, 8.0, 1.0)))
+    w = latent_weights(rng, W, H, d, r, dv, R)
+    h = bf16_round(rng.normal(size=(T, W)))
+    h[2] *= 6.0
+    nq = H * (d + r)
+    proj = h @ np.concatenate([w["m.q"], w["m.dkv"]]).T
+    inv, tab, mag = rotation_inputs(m["rot"], 100)
+    table, n_pages = paged(rng, T, P)
+    pool = torch.full((n_pages, P, 2 * R + r), float("nan"), device="cuda", dtype=torch.bfloat16)      # rows never written hold anything
+    pos = np.arange(T, dtype=np.int32)
+    slots = np.zeros(T, dtype=np.int32)
+    pj = dev(proj)
+    cut = 37
+    for lo, hi in ((0, cut), (cut, T)):
+        ops.latent_prep(pj[lo:hi], dev(w["m.dkv.norm"]), inv, tab, dev(pos[lo:hi], torch.int32), dev(slots[lo:hi], torch.int32),
+                        dev(table, torch.int32), pool, nq, eps, H, d, r, R, r, mag)
+    flat = f64(pool).reshape(n_pages, -1)
+    for t in (0, 1, P - 1, P, cut, T - 1):                  # the transposed latents are the rows' latents
+        pg = flat[table[0, t // P]]
+        assert np.array_equal(pg[:P * (R + r)].reshape(P, R + r)[t % P, :R], pg[P * (R + r):].reshape(R, P)[:, t % P]), t
+    if window:
+        want = np.zeros((T, H, dv))
+        q = proj[:, :nq].reshape(T, H, d + r)
+        c = bf16_round(plain.rms_unit(proj[:, nq:nq + R], eps) * w["m.dkv.norm"])
+        kr = bf16_round(plain.rotate_half(proj[:, nq + R:], pos, m["rot"]))
+        qr = plain.rotate_half(q[:, :, d:], pos, m["rot"])
+        vis = plain.window_mask(T, window)
+        for hd in range(H):
+            sc = (q[:, hd, :d] @ (c @ w["m.uk"][hd * d:(hd + 1) * d].T).T + qr[:, hd] @ kr.T) * m["scale"]
+            want[:, hd] = plain.softmax_rows(sc, vis, float(w["m.sink"][hd])) @ (c @ w["m.uv"][hd * dv:(hd + 1) * dv].T)
+    else:
+        want = plain.latent_attention(h, w, "m", m, eps).reshape(T, H, dv)
+    uk, uv = dev(w["m.uk"], torch.bfloat16), dev(w["m.uv"], torch.bfloat16)
+    uk_t = torch.empty(H * R, d, device="cuda", dtype=torch.bfloat16)
+    ops.latent_transpose(uk, uk_t, H)
+    assert torch.equal(uk_t.reshape(H, R, d), uk.reshape(H, d, R).transpose(1, 2))
+    args = (pj, uk, uv, dev(w["m.sink"]), pool, dev(table, torch.int32), dev(pos, torch.int32), dev(slots, torch.int32))
+    sizes = (H, d, r, R, dv, m["scale"], window)
+    bound = 4e-2 * max(1.0, np.abs(want).max())
+    slow = torch.zeros(T, H * dv, device="cuda", dtype=torch.bfloat16)
+    ops.latent_attention(*args, slow, *sizes)
+    err = np.abs(f64(slow).reshape(T, H, dv) - want)
+    assert err.max() < bound, ("rows", np.unravel_index(err.argmax(), err.shape), err.max())
+    entries = dev([[0, T, 0, 0]], torch.int32)
+    tiles = dev([[0, r0, min(64, T - r0)] for r0 in range(0, T, 64)], torch.int32)
+    ops.count_calls(True)
+    for lists in (dict(tiles=tiles, entries=entries), dict(all_rows=True), dict(all_rows=True, context=T),
+                  dict(tiles=tiles[:1], entries=entries, rows=dev(list(range(64, T)), torch.int32))):
+        fast = torch.zeros(T, H * dv, device="cuda", dtype=torch.bfloat16)
+        ops.latent_attention(*args, fast, *sizes, w_uk_t=uk_t, **lists)
+        err = np.abs(f64(fast).reshape(T, H, dv) - want)
+        assert err.max() < bound, (list(lists), np.unravel_index(err.argmax(), err.shape), err.max())
+    ops.force_decode_splits = 3
+    fast = torch.zeros(T, H * dv, device="cuda", dtype=torch.bfloat16)
+    ops.latent_attention(*args, fast, *sizes, w_uk_t=uk_t, all_rows=True, context=T)
+    ops.force_decode_splits = 0
+    err = np.abs(f64(fast).reshape(T, H, dv) - want)
+    assert err.max() < bound, ("split", np.unravel_index(err.argmax(), err.shape), err.max())
+    took = [c["name"] for c in ops.timing_report() if "latent_attention" in c["name"]]
+    ops.count_calls(False)
+    assert took and all("[mfma]" in n for n in took), took
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_router_over_the_chosen_and_clamped_experts(ops, dtype):
     rng = np.random.default_rng(11)

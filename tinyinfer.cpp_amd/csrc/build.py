@@ -37,6 +37,7 @@ HEADERS = ["common.h", "qk_prep.h", "tinyinfer_kernels.h", "tinyinfer_kernels_tu
 EXTRA_FLAGS: Dict[str, List[str]] = {
     "attention_bf16": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
     "diff_attention_bf16": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+    "latent_attention_bf16": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
 }
 
 def _discover() -> Dict[str, str]:
@@ -54,7 +55,7 @@ ON_DEMAND = ("measure",)
 # library serves them all
 ONLY_FOR = {"pointwise": ("Miterax", "Nazorax"), "recurrent": ("Miterax",), "residual": ("Mumasun",), "diff_attention": ("Mumasun",),
             "diff_attention_bf16": ("Mumasun",), "moe": ("Mumasun", "Nazorax"), "moe_bf16": ("Mumasun", "Nazorax"),
-            "latent_attention": ("Nazorax",)}
+            "latent_attention": ("Nazorax",), "latent_attention_bf16": ("Nazorax",)}
 # ... and libraries that a named architecture never calls into
 NOT_FOR = {"attention_generic": ("Mumasun",), "attention_bf16": ("Mumasun",)}
 

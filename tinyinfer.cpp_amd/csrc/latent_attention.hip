@@ -7,7 +7,8 @@
 // its value is the first R entries of the same row, and W_uv maps the head's weighted latent to its output.  The softmax
 // may hold a sink: exp(sink_h) in the denominator, with no key and no value.
 //
-//   latent_prep     proj f32 -> cache row [rms-normed c * w | rotated kr] (T), the heads' q_rot rotated in place
+//   latent_prep     proj f32 -> cache row [rms-normed c * w | rotated kr] (T), the heads' q_rot rotated in place; a page of
+//                   P (2 R + r) elements also gets the latents transposed [R][P] behind its rows (the matrix-core kernels' operand)
 //   latent_absorb   qa f32 [M, H, R + r] = [W_uk_h^T q_plain | q_rot]
 //   latent_rows     o f32 [M, H, R]: a workgroup per (row, head) over the paged rows, scores and softmax in 32-bit
 //   latent_expand   out T [M, H dv] = W_uv_h o
@@ -37,7 +38,7 @@ __global__ void __launch_bounds__(256)
 latent_prep_kernel(float* __restrict__ proj, int ldp, int off_kv, const float* __restrict__ norm_w, float eps,
                    const float* __restrict__ inv_freq, const float* __restrict__ rope_table, int table_len, float mag, int rot_dims,
                    const int* __restrict__ pos, const int* __restrict__ slot, const int* __restrict__ table, int table_stride,
-                   T* __restrict__ pool, int H, int d, int r, int R, int P) {
+                   T* __restrict__ pool, size_t page_elems, int H, int d, int r, int R, int P) {
   __shared__ float red[4];
   const int m = blockIdx.x;
   const int p = pos[m];
@@ -48,10 +49,16 @@ latent_prep_kernel(float* __restrict__ proj, int ldp, int off_kv, const float* _
   ss = block_sum<256>(ss, red);
   const float scale = 1.0f / sqrtf(ss / (float)R + eps);
   const int page = table[(size_t)slot[m] * table_stride + p / P];
-  T* dst = pool + ((size_t)max(page, 0) * P + p % P) * (R + r);
+  T* dst = pool + (size_t)max(page, 0) * page_elems + (size_t)(p % P) * (R + r);
+  // a page that is longer than its P rows holds the latents a second time, transposed [R][P], behind them
+  T* tdst = page_elems >= (size_t)P * (2 * R + r) ? pool + (size_t)max(page, 0) * page_elems + (size_t)P * (R + r) + p % P : nullptr;
   const int half = inv_freq ? rot_dims / 2 : 0;
   if (page >= 0) {      // the host reserves pages first; never write astray
-    for (int i = threadIdx.x; i < R; i += 256) st<T>(dst + i, c[i] * scale * norm_w[i]);
+    for (int i = threadIdx.x; i < R; i += 256) {
+      const float v = c[i] * scale * norm_w[i];
+      st<T>(dst + i, v);
+      if (tdst) st<T>(tdst + (size_t)i * P, v);
+    }
     const float* kr = c + R;
     for (int i = threadIdx.x; i < r; i += 256) {
       if (i >= half && i < 2 * half) continue;
@@ -79,15 +86,16 @@ latent_prep_kernel(float* __restrict__ proj, int ldp, int off_kv, const float* _
 
 extern "C" int ti_latent_prep(int dtype, float* proj, int ldp, int off_kv, const float* norm_w, float eps, const float* inv_freq,
                               const float* rope_table, int table_len, float mag, int rot_dims, const int* pos, const int* slot,
-                              const int* table, int table_stride, void* pool, int M, int H, int d, int r, int R, int page_size,
-                              hipStream_t stream) {
-  TI_REQUIRE(H > 0 && d >= 0 && r >= 0 && R > 0 && page_size > 0 && table_stride > 0 && off_kv >= H * (d + r) && ldp >= off_kv + R + r,
-             "latent_prep: bad sizes heads=%d dim=%d rot=%d rank=%d ld=%d", H, d, r, R, ldp);
+                              const int* table, int table_stride, void* pool, long page_elems, int M, int H, int d, int r, int R,
+                              int page_size, hipStream_t stream) {
+  TI_REQUIRE(H > 0 && d >= 0 && r >= 0 && R > 0 && page_size > 0 && table_stride > 0 && off_kv >= H * (d + r) && ldp >= off_kv + R + r &&
+                 page_elems >= (long)page_size * (R + r),
+             "latent_prep: bad sizes heads=%d dim=%d rot=%d rank=%d ld=%d page=%ld", H, d, r, R, ldp, page_elems);
   TI_REQUIRE(!inv_freq || (rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= r), "latent_prep: %d rotated entries do not fit %d", rot_dims, r);
   if (M == 0) return 0;
 #define LATENT_PREP(T)                                                                                                              \
   latent_prep_kernel<T><<<M, 256, 0, stream>>>(proj, ldp, off_kv, norm_w, eps, inv_freq, rope_table, table_len, mag, rot_dims, pos, \
-                                               slot, table, table_stride, (T*)pool, H, d, r, R, page_size)
+                                               slot, table, table_stride, (T*)pool, (size_t)page_elems, H, d, r, R, page_size)
   if (dtype == TI_F32) LATENT_PREP(float);
   else if (dtype == TI_BF16) LATENT_PREP(bf16_t);
   else TI_REQUIRE(false, "latent_prep: unknown dtype %d", dtype);
@@ -159,7 +167,7 @@ template <typename T, int DPL>
 __global__ void __launch_bounds__(256)
 latent_rows_kernel(const float* __restrict__ qa, const T* __restrict__ pool, const int* __restrict__ table, int table_stride,
                    const int* __restrict__ pos, const int* __restrict__ slot, const float* __restrict__ sink, float* __restrict__ out,
-                   int H, int R, int r, int P, float scale, int window) {
+                   int H, int R, int r, int P, size_t page_elems, float scale, int window) {
   extern __shared__ float s_o[];      // [groups][R]
   __shared__ float s_m[LA_GROUPS], s_l[LA_GROUPS];
   const int m = blockIdx.x, h = blockIdx.y;
@@ -180,7 +188,7 @@ latent_rows_kernel(const float* __restrict__ qa, const T* __restrict__ pool, con
   for (int p = lo + g; p <= p_q; p += LA_GROUPS) {
     const int page = tab[p / P];
     if (page < 0) continue;
-    const T* kp = pool + ((size_t)page * P + p % P) * DK;
+    const T* kp = pool + (size_t)page * page_elems + (size_t)(p % P) * DK;
     float kv[DPL];
     float s = 0.f;
 #pragma unroll
@@ -227,13 +235,13 @@ latent_rows_kernel(const float* __restrict__ qa, const T* __restrict__ pool, con
 }
 
 template <typename T>
-static int launch_latent_rows(int dpl, dim3 grid, size_t lds, const float* qa, const void* pool, const int* table, int table_stride,
+static int launch_latent_rows(int dpl, dim3 grid, size_t lds, const float* qa, const void* pool, size_t page_elems, const int* table, int table_stride,
                               const int* pos, const int* slot, const float* sink, float* out, int H, int R, int r, int P, float scale,
                               int window, hipStream_t stream) {
 #define LA_CASE(D)                                                                                                               \
   if (dpl <= D) {                                                                                                                \
     latent_rows_kernel<T, D><<<grid, 256, lds, stream>>>(qa, (const T*)pool, table, table_stride, pos, slot, sink, out, H, R, r, \
-                                                         P, scale, window);                                                      \
+                                                         P, page_elems, scale, window);                                                      \
     return 0;                                                                                                                    \
   }
   LA_CASE(2) LA_CASE(4) LA_CASE(8) LA_CASE(12) LA_CASE(16) LA_CASE(24) LA_CASE(32) LA_CASE(40) LA_CASE(48)
@@ -242,21 +250,22 @@ static int launch_latent_rows(int dpl, dim3 grid, size_t lds, const float* qa, c
 }
 
 // qa f32 [M, H, R + r]; pool T [pages][P][R + r]; sink f32 [H] (null: none); out f32 [M, H, R]
-extern "C" int ti_latent_attention_rows(int dtype, const float* qa, const void* pool, const int* table, int table_stride,
+extern "C" int ti_latent_attention_rows(int dtype, const float* qa, const void* pool, long page_elems, const int* table, int table_stride,
                                         const int* pos, const int* slot, const float* sink, float* out, int M, int H, int R, int r,
                                         int page_size, float scale, int window, hipStream_t stream) {
   TI_REQUIRE(H > 0 && H <= 65535 && R > 0 && r >= 0 && R + r <= 48 * LA_LANES, "latent_attention: heads=%d, a latent of %d + %d is not served (up to %d)",
              H, R, r, 48 * LA_LANES);
-  TI_REQUIRE(page_size > 0 && table_stride > 0, "latent_attention: bad page_size %d / table_stride %d", page_size, table_stride);
+  TI_REQUIRE(page_size > 0 && table_stride > 0 && page_elems >= (long)page_size * (R + r), "latent_attention: bad page_size %d / table_stride %d / page of %ld", page_size,
+             table_stride, page_elems);
   if (M == 0) return 0;
   const dim3 grid(M, H);
   const int dpl = (R + r + LA_LANES - 1) / LA_LANES;
   const size_t lds = (size_t)LA_GROUPS * R * 4;
   int rc;
   if (dtype == TI_F32)
-    rc = launch_latent_rows<float>(dpl, grid, lds, qa, pool, table, table_stride, pos, slot, sink, out, H, R, r, page_size, scale, window, stream);
+    rc = launch_latent_rows<float>(dpl, grid, lds, qa, pool, (size_t)page_elems, table, table_stride, pos, slot, sink, out, H, R, r, page_size, scale, window, stream);
   else if (dtype == TI_BF16)
-    rc = launch_latent_rows<bf16_t>(dpl, grid, lds, qa, pool, table, table_stride, pos, slot, sink, out, H, R, r, page_size, scale, window, stream);
+    rc = launch_latent_rows<bf16_t>(dpl, grid, lds, qa, pool, (size_t)page_elems, table, table_stride, pos, slot, sink, out, H, R, r, page_size, scale, window, stream);
   else
     TI_REQUIRE(false, "latent_attention: unknown dtype %d", dtype);
   TI_REQUIRE(rc == 0, "latent_attention: no kernel for a latent of %d + %d", R, r);
@@ -307,6 +316,26 @@ extern "C" int ti_latent_expand(int dtype, const float* o, const void* w_uv, voi
   if (dtype == TI_F32) latent_expand_kernel<float><<<grid, 256, lds, stream>>>(o, (const float*)w_uv, (float*)out, M, H, R, dv);
   else if (dtype == TI_BF16) latent_expand_kernel<bf16_t><<<grid, 256, lds, stream>>>(o, (const bf16_t*)w_uv, (bf16_t*)out, M, H, R, dv);
   else TI_REQUIRE(false, "latent_expand: unknown dtype %d", dtype);
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------------------------------ a head's matrices transposed
+// dst [H][cols][rows] = src [H][rows][cols]^T, head by head: what the matrix-core kernel of the absorbed query reads
+template <typename T>
+__global__ void __launch_bounds__(256)
+latent_transpose_kernel(const T* __restrict__ src, T* __restrict__ dst, int rows, int cols) {
+  const size_t base = (size_t)blockIdx.y * rows * cols;
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  if (e < rows * cols) dst[base + (size_t)(e % cols) * rows + e / cols] = src[base + e];
+}
+
+extern "C" int ti_latent_transpose(int dtype, const void* src, void* dst, int H, int rows, int cols, hipStream_t stream) {
+  TI_REQUIRE(H > 0 && H <= 65535 && rows > 0 && cols > 0, "latent_transpose: bad sizes %d x %d x %d", H, rows, cols);
+  const dim3 grid((rows * cols + 255) / 256, H);
+  if (dtype == TI_F32) latent_transpose_kernel<float><<<grid, 256, 0, stream>>>((const float*)src, (float*)dst, rows, cols);
+  else if (dtype == TI_BF16) latent_transpose_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)src, (bf16_t*)dst, rows, cols);
+  else TI_REQUIRE(false, "latent_transpose: unknown dtype %d", dtype);
   TI_LAUNCH_CHECK();
   return 0;
 }

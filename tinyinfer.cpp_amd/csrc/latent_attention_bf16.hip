@@ -1,0 +1,468 @@
+// Latent attention in bfloat16 on the matrix cores of gfx950.
+//
+// A token's page row holds [c (R) | kr (r)], and the page holds the latents a second time transposed, [R][P], behind its P
+// rows: the first product reduces over the R + r entries of a row, the second over the keys, and each reads its operand
+// along the dimension it reduces over, straight from memory.  Every head attends over the same rows with its absorbed
+// query qa = [W_uk^T q_plain | q_rot]; the weighted latent o goes through W_uv afterwards:
+//   latent_absorb_mfma   qa^T (R x 16 tokens)   = W_uk_h^T (R x d) . q_plain^T      one workgroup per (16 tokens, head)
+//   S^T (16 keys x 16 columns)                   = [c | kr] (16 x DK) . qa^T
+//   O^T (R x 16 columns)                        += c^T (R x 32 keys) . P^T
+//   latent_expand_mfma   out^T (dv x 16 tokens)  = W_uv_h (dv x R) . o^T
+// all with v_mfma_f32_16x16x32_bf16.  The transposed score tile leaves each lane with four keys of one column, the layout
+// the second product wants for P^T.  Scores, the running softmax and the sink (exp(sink_h) in the denominator only, added
+// once when a column is finished) are 32-bit.
+//
+// What the 16 columns are: for a tile of a prompt's portion, 16 consecutive tokens of one head (a workgroup's four
+// wavefronts take four such runs); for single rows (decoded tokens), 16 heads of one token, the four wavefronts taking the
+// pairs of key blocks in turns and merging through LDS, and several workgroups sharing a long context with a merge kernel
+// behind them.  A column at position p sees the keys max(0, p - window + 1) .. p (window 0: all).
+//
+// Sizes: the kernels are compiled for (k-steps of 32 over R + r, blocks of 16 over R) = (3, 4), (6, 8), (10, 16), (18, 32);
+// a model takes the smallest that holds it, steps and blocks beyond its sizes are skipped.  R a multiple of 16, R + r and
+// the unrotated query size multiples of 8, the value size a multiple of 16, pages of a multiple of 16 rows.
+#include "common.h"
+#include "tinyinfer_kernels.h"
+
+TI_ERROR_API
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+
+#define LA_LOG2E 1.4426950408889634f
+
+union LFrag8 {
+  uint4 u;
+  bf16x8 v;
+};
+
+struct LatPages {
+  const bf16_t* pool;   // [pages][rows: [P][DK] | transposed latents: [R][P]]
+  const int* table;     // block-table row of the request
+  int P, DK, R;
+  size_t page_elems;
+};
+
+template <int NRT>
+struct LatState {
+  float m, l;           // maximum (units of log 2) of the column; this lane's share of the sum of weights
+  floatx4 o[NRT];       // O^T: rows (latent entries) 16 d + 4 (lane / 16) + i, column lane % 16
+  __device__ __forceinline__ void clear() {
+    m = -INFINITY;
+    l = 0.f;
+#pragma unroll
+    for (int d = 0; d < NRT; ++d) o[d] = floatx4{0.f, 0.f, 0.f, 0.f};
+  }
+};
+
+// One pair of blocks of 16 keys, [keyA, keyA + 16) and [keyA + 16, keyA + 32), for this wavefront's 16 columns.
+//   qf        qa^T fragments: column lane % 16, entries 32 s + 8 (lane / 16) .. + 7
+//   lo, hi    the keys this lane's column sees: lo <= key <= hi (lo > hi: none)
+//   lo_max, hi_min   the largest lo and the smallest hi of the wavefront's live columns
+//   kv_last   last position of the request that has been written (rows after it hold anything, NaN included)
+//   safe_key  a key whose page exists: loads of blocks that do not count go there, so that they never leave the pool
+template <int NKS, int NRT>
+__device__ __forceinline__ void latent_pair(const LatPages& kv, const LFrag8* qf, int keyA, int lo, int hi, int lo_max, int hi_min,
+                                            int kv_last, int safe_key, float scale2, LatState<NRT>& st) {
+  const int lane = threadIdx.x & 63;
+  const int r16 = lane & 15, quad = lane >> 4;
+  const int keyB = keyA + 16;
+  int pageA = keyA <= kv_last ? kv.table[keyA / kv.P] : -1;
+  int pageB = keyB <= kv_last ? kv.table[keyB / kv.P] : -1;
+  const bool validA = pageA >= 0, validB = pageB >= 0;
+  int rowA = keyA % kv.P, rowB = keyB % kv.P;
+  if (!validA) {
+    pageA = kv.table[safe_key / kv.P];
+    rowA = (safe_key % kv.P) & ~15;
+  }
+  if (!validB) {
+    pageB = kv.table[safe_key / kv.P];
+    rowB = (safe_key % kv.P) & ~15;
+  }
+  const bool plain = validA && validB && keyA >= lo_max && keyB + 15 <= hi_min;
+  const bf16_t* ka = kv.pool + (size_t)pageA * kv.page_elems + (size_t)(rowA + r16) * kv.DK + quad * 8;
+  const bf16_t* kb = kv.pool + (size_t)pageB * kv.page_elems + (size_t)(rowB + r16) * kv.DK + quad * 8;
+  floatx4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int s = 0; s < NKS; ++s) {
+    if (s * 32 < kv.DK) {
+      LFrag8 a, b;
+      a.u = b.u = make_uint4(0u, 0u, 0u, 0u);
+      if (s * 32 + quad * 8 < kv.DK) {
+        a.u = *reinterpret_cast<const uint4*>(ka + s * 32);
+        b.u = *reinterpret_cast<const uint4*>(kb + s * 32);
+      }
+      sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qf[s].v, sa, 0, 0, 0);
+      sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b.v, qf[s].v, sb, 0, 0, 0);
+    }
+  }
+  float sv[8];
+  unsigned keepA[2] = {0xFFFFFFFFu, 0xFFFFFFFFu}, keepB[2] = {0xFFFFFFFFu, 0xFFFFFFFFu};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int ja = keyA + quad * 4 + i, jb = keyB + quad * 4 + i;
+    const bool see_a = plain || (validA & (ja >= lo) & (ja <= hi));
+    const bool see_b = plain || (validB & (jb >= lo) & (jb <= hi));
+    sv[i] = see_a ? sa[i] * scale2 : -INFINITY;
+    sv[4 + i] = see_b ? sb[i] * scale2 : -INFINITY;
+    if (!plain) {
+      // 0 * NaN is NaN: latents of rows that were never written (or of a stand-in page) become zero
+      const unsigned half = (i & 1) ? 0x0000FFFFu : 0xFFFF0000u;
+      if (!validA | (ja > kv_last)) keepA[i >> 1] &= half;
+      if (!validB | (jb > kv_last)) keepB[i >> 1] &= half;
+    }
+  }
+  float bm = sv[0];
+#pragma unroll
+  for (int i = 1; i < 8; ++i) bm = fmaxf(bm, sv[i]);
+  bm = fmaxf(bm, __shfl_xor(bm, 16, 64));
+  bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
+  const float m_new = fmaxf(st.m, bm);
+  const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+  float pv[8], ps = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    pv[i] = __builtin_amdgcn_exp2f(sv[i] - m_safe);
+    ps += pv[i];
+  }
+  LFrag8 pf;
+  pf.u = make_uint4(pack_bf16x2(pv[0], pv[1]), pack_bf16x2(pv[2], pv[3]), pack_bf16x2(pv[4], pv[5]), pack_bf16x2(pv[6], pv[7]));
+  if (__builtin_amdgcn_ballot_w64(m_new != st.m) != 0) {
+    const float alpha = __builtin_amdgcn_exp2f(st.m - m_safe);      // m = -inf: 0, and l and o are 0 anyway
+    st.l *= alpha;
+#pragma unroll
+    for (int d = 0; d < NRT; ++d)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) st.o[d][i] *= alpha;
+    st.m = m_new;
+  }
+  st.l += ps;
+  // the transposed latents: row (entry) 16 d + lane % 16, keys 4 (lane / 16) .. + 3 of either block
+  const size_t t_base = (size_t)kv.P * kv.DK;
+  const bf16_t* va = kv.pool + (size_t)pageA * kv.page_elems + t_base + (size_t)r16 * kv.P + rowA + quad * 4;
+  const bf16_t* vb = kv.pool + (size_t)pageB * kv.page_elems + t_base + (size_t)r16 * kv.P + rowB + quad * 4;
+  const unsigned v_step = 16u * kv.P;
+#pragma unroll
+  for (int d = 0; d < NRT; ++d) {
+    if (d * 16 < kv.R) {
+      const uint2 a = *reinterpret_cast<const uint2*>(va + d * v_step);
+      const uint2 b = *reinterpret_cast<const uint2*>(vb + d * v_step);
+      LFrag8 v;
+      v.u = make_uint4(a.x & keepA[0], a.y & keepA[1], b.x & keepB[0], b.y & keepB[1]);
+      st.o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v.v, pf.v, st.o[d], 0, 0, 0);
+    }
+  }
+}
+
+// the absorbed query of this lane's column: qa row [DK], entries 32 s + 8 (lane / 16) .. + 7
+template <int NKS>
+__device__ __forceinline__ void load_query(const bf16_t* qrow, int DK, LFrag8* qf) {
+  const int quad = (threadIdx.x & 63) >> 4;
+#pragma unroll
+  for (int s = 0; s < NKS; ++s) {
+    qf[s].u = make_uint4(0u, 0u, 0u, 0u);
+    if (s * 32 + quad * 8 < DK) qf[s].u = *reinterpret_cast<const uint4*>(qrow + s * 32 + quad * 8);
+  }
+}
+
+// the column's weighted latent divided by its sum of weights, the sink in the sum: o bf16 [R] of the column
+template <int NRT>
+__device__ __forceinline__ void finish_column(LatState<NRT>& st, const float* sink, int h, int R, bf16_t* dst, bool live) {
+  const int quad = (threadIdx.x & 63) >> 4;
+  float l = st.l;
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  const float s2 = sink ? sink[h] * LA_LOG2E : -INFINITY;
+  const float mm = fmaxf(st.m, s2);
+  const float m_safe = (mm == -INFINITY) ? 0.f : mm;
+  const float a = __builtin_amdgcn_exp2f(st.m - m_safe);
+  const float lt = l * a + (sink ? __builtin_amdgcn_exp2f(s2 - m_safe) : 0.f);
+  const float f = lt > 0.f ? a / lt : 0.f;
+  if (!live) return;
+#pragma unroll
+  for (int d = 0; d < NRT; ++d)
+    if (d * 16 < R)
+      *reinterpret_cast<uint2*>(dst + d * 16 + quad * 4) =
+          make_uint2(pack_bf16x2(st.o[d][0] * f, st.o[d][1] * f), pack_bf16x2(st.o[d][2] * f, st.o[d][3] * f));
+}
+
+// ------------------------------------------------------------------------------------------ tiles of a portion
+// tiles int32 [n][3] = (entry, first row, rows <= 64); entries int32 [.][4] = (row0, tokens, start, -).  qa [M][H][DK],
+// o [M][H][R].  Grid (tiles, heads), four wavefronts of 16 rows each.
+template <int NKS, int NRT>
+__global__ void __launch_bounds__(256)
+latent_tiles_kernel(const bf16_t* __restrict__ qa, const bf16_t* __restrict__ pool, const int* __restrict__ table, int table_stride,
+                    const int* __restrict__ tiles, const int* __restrict__ entries, const float* __restrict__ sink,
+                    bf16_t* __restrict__ o, int H, int R, int DK, int P, size_t page_elems, float scale2, int window) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r16 = lane & 15;
+  const int e = tiles[3 * blockIdx.x], row0 = tiles[3 * blockIdx.x + 1] + 16 * wave;
+  const int n_rows = tiles[3 * blockIdx.x + 2] - 16 * wave;
+  if (n_rows <= 0) return;
+  const int h = blockIdx.y;
+  const int e_row0 = entries[4 * e], e_n = entries[4 * e + 1], e_start = entries[4 * e + 2];
+  const int kv_last = e_start + e_n - 1;
+  const bool live = r16 < n_rows;
+  const int row = row0 + (live ? r16 : 0);
+  const int p = e_start + (row - e_row0);
+  const int lo_p = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  const int lo = live ? lo_p : 1, hi = live ? p : 0;
+  int lo_min = live ? lo : 0x7fffffff, lo_max = live ? lo : 0, hi_min = live ? hi : 0x7fffffff, hi_max = hi;
+#pragma unroll
+  for (int x = 1; x < 16; x <<= 1) {
+    lo_min = min(lo_min, __shfl_xor(lo_min, x, 64));
+    lo_max = max(lo_max, __shfl_xor(lo_max, x, 64));
+    hi_min = min(hi_min, __shfl_xor(hi_min, x, 64));
+    hi_max = max(hi_max, __shfl_xor(hi_max, x, 64));
+  }
+  LatPages kv{pool, table + (size_t)e * table_stride, P, DK, R, page_elems};
+  LFrag8 qf[NKS];
+  load_query<NKS>(qa + ((size_t)row * H + h) * DK, DK, qf);
+  LatState<NRT> st;
+  st.clear();
+  for (int pr = lo_min / 32; pr <= hi_max / 32; ++pr)
+    latent_pair<NKS, NRT>(kv, qf, pr * 32, lo, hi, lo_max, hi_min, kv_last, hi_max, scale2, st);
+  finish_column<NRT>(st, sink, h, R, o + ((size_t)row * H + h) * R, live);
+}
+
+// ------------------------------------------------------------------------------------------ single rows
+// rows int32 [n] (null: row r is r); the 16 columns are the heads 16 blockIdx.y .. + 15 of the row's token.  Workgroup z of
+// gridDim.z, wavefront v take the pairs of blocks 4 z + v, 4 z + v + 4 gridDim.z, ...; the wavefronts merge through LDS in
+// the order 1, 2, 3.  One workgroup a row finishes the columns; several leave their shares in `part`.
+template <int NRT>
+__device__ __forceinline__ void merge_share(LatState<NRT>& st, const float* src, int lane) {
+  const float m2 = src[NRT * 4 * 64 + lane], l2 = src[(NRT * 4 + 1) * 64 + lane];
+  const float mm = fmaxf(st.m, m2);
+  const float m_safe = (mm == -INFINITY) ? 0.f : mm;
+  const float a = __builtin_amdgcn_exp2f(st.m - m_safe), b = __builtin_amdgcn_exp2f(m2 - m_safe);
+  st.l = st.l * a + l2 * b;
+#pragma unroll
+  for (int d = 0; d < NRT; ++d)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) st.o[d][i] = st.o[d][i] * a + src[(d * 4 + i) * 64 + lane] * b;
+  st.m = mm;
+}
+
+template <int NRT>
+__device__ __forceinline__ void store_share(const LatState<NRT>& st, float* dst, int lane) {
+#pragma unroll
+  for (int d = 0; d < NRT; ++d)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dst[(d * 4 + i) * 64 + lane] = st.o[d][i];
+  dst[NRT * 4 * 64 + lane] = st.m;
+  dst[(NRT * 4 + 1) * 64 + lane] = st.l;
+}
+
+template <int NKS, int NRT>
+__global__ void __launch_bounds__(256)
+latent_rows_mfma_kernel(const bf16_t* __restrict__ qa, const bf16_t* __restrict__ pool, const int* __restrict__ table, int table_stride,
+                        const int* __restrict__ pos, const int* __restrict__ slot, const int* __restrict__ rows,
+                        const float* __restrict__ sink, bf16_t* __restrict__ o, int H, int R, int DK, int P, size_t page_elems,
+                        float scale2, int window, float* __restrict__ part, int n_splits) {
+  extern __shared__ float lds[];     // [NRT 4 + 2][64]
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r16 = lane & 15;
+  const int m = rows ? rows[blockIdx.x] : blockIdx.x;
+  const int p = pos[m];
+  const bool live = (int)blockIdx.y * 16 + r16 < H;
+  const int h = live ? blockIdx.y * 16 + r16 : 0;
+  const int lo_all = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  const int lo = live ? lo_all : 1, hi = live ? p : 0;
+  LatPages kv{pool, table + (size_t)slot[m] * table_stride, P, DK, R, page_elems};
+  LFrag8 qf[NKS];
+  load_query<NKS>(qa + ((size_t)m * H + h) * DK, DK, qf);
+  LatState<NRT> st;
+  st.clear();
+  for (int pr = lo_all / 32 + 4 * blockIdx.z + wave; pr <= p / 32; pr += 4 * n_splits)
+    latent_pair<NKS, NRT>(kv, qf, pr * 32, lo, hi, lo_all, p, p, p, scale2, st);
+  for (int w = 1; w < 4; ++w) {
+    if (wave == w) store_share<NRT>(st, lds, lane);
+    __syncthreads();
+    if (wave == 0) merge_share<NRT>(st, lds, lane);
+    __syncthreads();
+  }
+  if (wave > 0) return;
+  if (n_splits == 1) {
+    finish_column<NRT>(st, sink, h, R, o + ((size_t)m * H + h) * R, live);
+    return;
+  }
+  store_share<NRT>(st, part + (((size_t)blockIdx.x * gridDim.y + blockIdx.y) * n_splits + blockIdx.z) * (NRT * 4 + 2) * 64, lane);
+}
+
+// one wavefront per (row, 16 heads): the shares of the workgroups that split the row's keys, in ascending order
+template <int NRT>
+__global__ void __launch_bounds__(64)
+latent_rows_merge_kernel(const float* __restrict__ part, const int* __restrict__ rows, const float* __restrict__ sink,
+                         bf16_t* __restrict__ o, int H, int R, int n_splits) {
+  const int lane = threadIdx.x, r16 = lane & 15;
+  const int m = rows ? rows[blockIdx.x] : blockIdx.x;
+  const bool live = (int)blockIdx.y * 16 + r16 < H;
+  const int h = live ? blockIdx.y * 16 + r16 : 0;
+  LatState<NRT> st;
+  st.clear();
+  for (int s = 0; s < n_splits; ++s)
+    merge_share<NRT>(st, part + (((size_t)blockIdx.x * gridDim.y + blockIdx.y) * n_splits + s) * (NRT * 4 + 2) * 64, lane);
+  finish_column<NRT>(st, sink, h, R, o + ((size_t)m * H + h) * R, live);
+}
+
+// ------------------------------------------------------------------------------------------ the absorbed query
+// qa [M][H][DK] bf16: entries c < R: sum_k q[m, h, k] W_uk[h d + k, c], from w_uk_t [H][R][d] (a head's matrix transposed);
+// entries R + j: q_rot[m, h, j].  proj f32 [M, ld] holds the heads' queries [d + r] from column 0.  Grid (tokens / 16, heads);
+// a wavefront takes the blocks of 16 latent entries wave, wave + 4, ...
+__global__ void __launch_bounds__(256)
+latent_absorb_mfma_kernel(const float* __restrict__ proj, int ldp, const bf16_t* __restrict__ w_uk_t, bf16_t* __restrict__ qa, int M,
+                          int H, int d, int r, int R) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r16 = lane & 15, quad = lane >> 4;
+  const int h = blockIdx.y, DK = R + r;
+  const int tok = blockIdx.x * 16 + r16;
+  const bool live = tok < M;
+  const float* q = proj + (size_t)(live ? tok : M - 1) * ldp + (size_t)h * (d + r);
+  for (int ct = wave; ct * 16 < R; ct += 4) {
+    const bf16_t* w = w_uk_t + ((size_t)h * R + ct * 16 + r16) * d + quad * 8;
+    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int k0 = 0; k0 < d; k0 += 32) {
+      LFrag8 a, b;
+      a.u = b.u = make_uint4(0u, 0u, 0u, 0u);
+      if (k0 + quad * 8 < d) {
+        a.u = *reinterpret_cast<const uint4*>(w + k0);
+        const float4 x = *reinterpret_cast<const float4*>(q + k0 + quad * 8), y = *reinterpret_cast<const float4*>(q + k0 + quad * 8 + 4);
+        b.u = make_uint4(pack_bf16x2(x.x, x.y), pack_bf16x2(x.z, x.w), pack_bf16x2(y.x, y.y), pack_bf16x2(y.z, y.w));
+      }
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc, 0, 0, 0);
+    }
+    if (live)
+      *reinterpret_cast<uint2*>(qa + ((size_t)tok * H + h) * DK + ct * 16 + quad * 4) =
+          make_uint2(pack_bf16x2(acc[0], acc[1]), pack_bf16x2(acc[2], acc[3]));
+  }
+  const int n = min(16, M - (int)blockIdx.x * 16);
+  for (int e = threadIdx.x; e < n * r; e += 256) {
+    const int t = blockIdx.x * 16 + e / r, j = e % r;
+    qa[((size_t)t * H + h) * DK + R + j] = f2bf(proj[(size_t)t * ldp + (size_t)h * (d + r) + d + j]);
+  }
+}
+
+// ------------------------------------------------------------------------------------------ a head's weighted latent to its output
+// out [M][H dv] bf16: out[m, h dv + j] = sum_c o[m, h, c] W_uv[h dv + j, c].  Grid (tokens / 16, heads); a wavefront takes the
+// blocks of 16 outputs wave, wave + 4, ...
+__global__ void __launch_bounds__(256)
+latent_expand_mfma_kernel(const bf16_t* __restrict__ o, const bf16_t* __restrict__ w_uv, bf16_t* __restrict__ out, int M, int H, int R,
+                          int dv) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r16 = lane & 15, quad = lane >> 4;
+  const int h = blockIdx.y;
+  const int tok = blockIdx.x * 16 + r16;
+  const bool live = tok < M;
+  const bf16_t* orow = o + ((size_t)(live ? tok : M - 1) * H + h) * R + quad * 8;
+  for (int jt = wave; jt * 16 < dv; jt += 4) {
+    const bf16_t* w = w_uv + ((size_t)h * dv + jt * 16 + r16) * R + quad * 8;
+    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int c0 = 0; c0 < R; c0 += 32) {
+      LFrag8 a, b;
+      a.u = b.u = make_uint4(0u, 0u, 0u, 0u);
+      if (c0 + quad * 8 < R) {
+        a.u = *reinterpret_cast<const uint4*>(w + c0);
+        b.u = *reinterpret_cast<const uint4*>(orow + c0);
+      }
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc, 0, 0, 0);
+    }
+    if (live)
+      *reinterpret_cast<uint2*>(out + (size_t)tok * H * dv + (size_t)h * dv + jt * 16 + quad * 4) =
+          make_uint2(pack_bf16x2(acc[0], acc[1]), pack_bf16x2(acc[2], acc[3]));
+  }
+}
+
+// ------------------------------------------------------------------------------------------ host
+extern "C" int ti_latent_bf16_served(int H, int d, int r, int R, int dv, int page_size) {
+  return H > 0 && d > 0 && d % 8 == 0 && (d + r) % 4 == 0 && r >= 0 && R > 0 && R % 16 == 0 && R <= 512 && (R + r) % 8 == 0 && R + r <= 576 && dv > 0 &&
+         dv % 16 == 0 && page_size > 0 && page_size % 16 == 0;
+}
+
+#define LA_DISPATCH(CALL)                                         \
+  do {                                                            \
+    if (DK <= 96 && R <= 64) { CALL(3, 4); }                      \
+    else if (DK <= 192 && R <= 128) { CALL(6, 8); }               \
+    else if (DK <= 320 && R <= 256) { CALL(10, 16); }             \
+    else { CALL(18, 32); }                                        \
+  } while (0)
+
+static int rows_block(int DK, int R) {
+  if (DK <= 96 && R <= 64) return 4;
+  if (DK <= 192 && R <= 128) return 8;
+  if (DK <= 320 && R <= 256) return 16;
+  return 32;
+}
+
+extern "C" int ti_latent_absorb_bf16(const float* proj, int ld, const void* w_uk_t, void* qa, int M, int H, int d, int r, int R,
+                                     hipStream_t stream) {
+  TI_REQUIRE(H > 0 && H <= 65535 && d > 0 && d % 8 == 0 && r >= 0 && R > 0 && R % 16 == 0 && ld >= H * (d + r) && ld % 4 == 0 &&
+                 (d + r) % 4 == 0,
+             "latent_absorb (bf16): bad sizes heads=%d dim=%d rot=%d rank=%d ld=%d", H, d, r, R, ld);
+  if (M == 0) return 0;
+  latent_absorb_mfma_kernel<<<dim3((M + 15) / 16, H), 256, 0, stream>>>(proj, ld, (const bf16_t*)w_uk_t, (bf16_t*)qa, M, H, d, r, R);
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int ti_latent_expand_bf16(const void* o, const void* w_uv, void* out, int M, int H, int R, int dv, hipStream_t stream) {
+  TI_REQUIRE(H > 0 && H <= 65535 && R > 0 && R % 8 == 0 && dv > 0 && dv % 16 == 0, "latent_expand (bf16): bad sizes heads=%d rank=%d vdim=%d", H, R, dv);
+  if (M == 0) return 0;
+  latent_expand_mfma_kernel<<<dim3((M + 15) / 16, H), 256, 0, stream>>>((const bf16_t*)o, (const bf16_t*)w_uv, (bf16_t*)out, M, H, R, dv);
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
+// pool bf16 [pages][P rows of R + r | R rows of P]: page_elems elements a page
+extern "C" int ti_latent_attention_tiles_bf16(const void* qa, const void* pool, long page_elems, const int* table, int table_stride,
+                                              const int* tiles, const int* entries, const float* sink, void* o, int n_tiles, int H,
+                                              int R, int r, int page_size, float scale, int window, hipStream_t stream) {
+  const int DK = R + r;
+  TI_REQUIRE(ti_latent_bf16_served(H, 8, 0, R, 16, page_size) && (R + r) % 8 == 0 && R + r <= 576 && H <= 65535 && table_stride > 0 && window >= 0 &&
+                 page_elems >= (long)page_size * (DK + R),
+             "latent_attention (tiles): heads=%d, a latent of %d + %d, pages of %d rows and %ld elements are not served", H, R, r,
+             page_size, page_elems);
+  if (n_tiles == 0) return 0;
+  const dim3 grid(n_tiles, H);
+#define LA_TILES(K, V)                                                                                                          \
+  latent_tiles_kernel<K, V><<<grid, 256, 0, stream>>>((const bf16_t*)qa, (const bf16_t*)pool, table, table_stride, tiles, entries, \
+                                                      sink, (bf16_t*)o, H, R, DK, page_size, (size_t)page_elems, scale * LA_LOG2E, window)
+  LA_DISPATCH(LA_TILES);
+#undef LA_TILES
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int ti_latent_attention_rows_bf16(const void* qa, const void* pool, long page_elems, const int* table, int table_stride,
+                                             const int* pos, const int* slot, const int* rows, const float* sink, void* o, int n_rows,
+                                             int H, int R, int r, int page_size, float scale, int window, float* part, int n_splits,
+                                             hipStream_t stream) {
+  const int DK = R + r;
+  TI_REQUIRE(ti_latent_bf16_served(H, 8, 0, R, 16, page_size) && (R + r) % 8 == 0 && R + r <= 576 && table_stride > 0 && window >= 0 && page_elems >= (long)page_size * (DK + R),
+             "latent_attention (rows): heads=%d, a latent of %d + %d, pages of %d rows and %ld elements are not served", H, R, r, page_size,
+             page_elems);
+  TI_REQUIRE(n_splits >= 1 && n_splits <= 64 && (n_splits == 1 || part), "latent_attention (rows): %d splits need scratch", n_splits);
+  if (n_rows == 0) return 0;
+  const int groups = (H + 15) / 16;
+  TI_REQUIRE(groups <= 65535, "latent_attention (rows): %d heads are not served", H);
+  const dim3 grid(n_rows, groups, n_splits);
+  const size_t lds = (size_t)(rows_block(DK, R) * 4 + 2) * 64 * 4;
+#define LA_ROWS(K, V)                                                                                                              \
+  latent_rows_mfma_kernel<K, V><<<grid, 256, lds, stream>>>((const bf16_t*)qa, (const bf16_t*)pool, table, table_stride, pos, slot, rows, \
+                                                            sink, (bf16_t*)o, H, R, DK, page_size, (size_t)page_elems, scale * LA_LOG2E, \
+                                                            window, part, n_splits)
+  LA_DISPATCH(LA_ROWS);
+#undef LA_ROWS
+  TI_LAUNCH_CHECK();
+  if (n_splits > 1) {
+    const dim3 mgrid(n_rows, groups);
+#define LA_MERGE(K, V) latent_rows_merge_kernel<V><<<mgrid, 64, 0, stream>>>(part, rows, sink, (bf16_t*)o, H, R, n_splits)
+    LA_DISPATCH(LA_MERGE);
+#undef LA_MERGE
+    TI_LAUNCH_CHECK();
+  }
+  return 0;
+}
+
+// floats of scratch for ti_latent_attention_rows_bf16 with n_splits > 1
+extern "C" long ti_latent_attention_rows_scratch(int n_rows, int H, int R, int r, int n_splits) {
+  return (long)n_rows * ((H + 15) / 16) * n_splits * (rows_block(R + r, R) * 4 + 2) * 64;
+}

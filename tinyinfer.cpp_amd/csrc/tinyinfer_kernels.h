@@ -135,21 +135,43 @@ int ti_concat_round(int out_dtype, const float* a, const float* b, void* out, in
 // its value W_uv c, neither ever formed per token)
 // proj f32 [M, ld]: queries [H][d + r] from column 0, [latent (R) | shared key part (r)] from column off_kv.  The latent is
 // RMS-normed (norm_w [R], eps) and goes with the rotated key part into the token's row of pool [pages][P][R + r]; the heads'
-// last r query entries are rotated in place.  Rotation as in ti_qkv_prep_write (rot_dims <= r)
+// last r query entries are rotated in place.  Rotation as in ti_qkv_prep_write (rot_dims <= r).  A page has page_elems
+// elements: with P (2 R + r) or more it also holds the latents transposed, [R][P], behind its P rows
 int ti_latent_prep(int dtype, float* proj, int ld, int off_kv, const float* norm_w, float eps, const float* inv_freq,
                    const float* rope_table, int table_len, float mag, int rot_dims, const int* pos, const int* slot,
-                   const int* table, int table_stride, void* pool, int M, int H, int d, int r, int R, int page_size,
+                   const int* table, int table_stride, void* pool, long page_elems, int M, int H, int d, int r, int R, int page_size,
                    hipStream_t stream);
 // qa f32 [M, H, R + r] = [W_uk_h^T q_h[:d] | q_h[d:]] with w_uk [H d][R] in `dtype`
 int ti_latent_absorb(int dtype, const float* proj, int ld, const void* w_uk, float* qa, int M, int H, int d, int r, int R,
                      hipStream_t stream);
 // o f32 [M, H, R] = sum_j p_j c_j over the row's visible positions (window <= 0: all up to its own), p the softmax of
 // (qa . [c_j | kr_j]) scale with exp(sink[h]) joining the denominator (sink null: none)
-int ti_latent_attention_rows(int dtype, const float* qa, const void* pool, const int* table, int table_stride, const int* pos,
+int ti_latent_attention_rows(int dtype, const float* qa, const void* pool, long page_elems, const int* table, int table_stride, const int* pos,
                              const int* slot, const float* sink, float* out, int M, int H, int R, int r, int page_size,
                              float scale, int window, hipStream_t stream);
 // out [M, H dv] = W_uv_h o[m, h] with w_uv [H dv][R], both in `dtype`
 int ti_latent_expand(int dtype, const float* o, const void* w_uv, void* out, int M, int H, int R, int dv, hipStream_t stream);
+// dst [H][cols][rows] = src [H][rows][cols] transposed head by head
+int ti_latent_transpose(int dtype, const void* src, void* dst, int H, int rows, int cols, hipStream_t stream);
+
+// ---- libti_latent_attention_bf16: the same on the matrix cores, over pages that hold the latents a second time transposed
+// 1 if the sizes are served (R % 16, (R + r) % 8, d % 8, (d + r) % 4, dv % 16, pages of a multiple of 16 rows, R <= 512, R + r <= 576)
+int ti_latent_bf16_served(int H, int d, int r, int R, int dv, int page_size);
+// qa bf16 [M, H, R + r] from w_uk_t bf16 [H][R][d] (ti_latent_transpose of w_uk)
+int ti_latent_absorb_bf16(const float* proj, int ld, const void* w_uk_t, void* qa, int M, int H, int d, int r, int R, hipStream_t stream);
+// o bf16 [M, H, R] for the tiles int32 [n][3] = (entry, first row, rows <= 64) of entries int32 [.][4] = (row0, tokens, start, -);
+// the block table's row of a tile is its entry's
+int ti_latent_attention_tiles_bf16(const void* qa, const void* pool, long page_elems, const int* table, int table_stride,
+                                   const int* tiles, const int* entries, const float* sink, void* o, int n_tiles, int H, int R, int r,
+                                   int page_size, float scale, int window, hipStream_t stream);
+// ... and for single rows (rows int32 [n], null: every row): 16 heads a wavefront; n_splits workgroups share a row's keys
+// (part: ti_latent_attention_rows_scratch floats)
+int ti_latent_attention_rows_bf16(const void* qa, const void* pool, long page_elems, const int* table, int table_stride, const int* pos,
+                                  const int* slot, const int* rows, const float* sink, void* o, int n_rows, int H, int R, int r,
+                                  int page_size, float scale, int window, float* part, int n_splits, hipStream_t stream);
+long ti_latent_attention_rows_scratch(int n_rows, int H, int R, int r, int n_splits);
+// out bf16 [M, H dv] = W_uv_h o[m, h] from o bf16 [M, H, R]
+int ti_latent_expand_bf16(const void* o, const void* w_uv, void* out, int M, int H, int R, int dv, hipStream_t stream);
 
 // ---- libti_recurrent: the mLSTM cell as a scan over each request's tokens of the step
 // proj f32 [M, ld] holds, from the columns off_* on, the heads' q and k [heads][dk], v [heads][dv] and the gates'

@@ -1263,9 +1263,27 @@ int ti_ops_call(void* ops_, const char* op_, const ti_tensor* t, int n_t, const 
     ops.latent_prep(arg(0), (int)num(0), arg(1), (float)num(1), r, iptr(4), iptr(5), view_of(6, arg(7)), arg(7), (int)num(2), (int)num(3),
                     (int)num(4), (int)num(5));
   } else if (op == "latent_attention") {
-    // proj, w_uk, w_uv, sink (may be absent), pool, table, positions, slots, out; heads, dim, rot_dim, rank, v_dim, scale, window
+    // proj, w_uk, w_uv, sink (may be absent), pool, table, positions, slots, out, [w_uk_t, tiles [n, 3], rows [n], entries [R, 4]];
+    // heads, dim, rot_dim, rank, v_dim, scale, window, [rows of single tokens where no list names them, their longest context]
+    Ops::LatentLists l;
+    const bool listed = n_t > 9 && arg(9).defined();
+    if (n_t > 10 && arg(10).defined()) {
+      l.tiles = iptr(10);
+      l.n_tiles = (int)arg(10).shape[0];
+    }
+    if (n_t > 11 && arg(11).defined()) {
+      l.rows = iptr(11);
+      l.n_rows = (int)arg(11).shape[0];
+    } else if (n_s > 7) {
+      l.n_rows = (int)num(7);
+    }
+    if (n_t > 12 && arg(12).defined()) l.entry_meta = iptr(12);
+    if (n_s > 8) l.context = (int)num(8);
     ops.latent_attention(arg(0), arg(1), arg(2), arg(3), arg(4), view_of(5, arg(4)), iptr(6), iptr(7), arg(8), (int)num(0), (int)num(1),
-                         (int)num(2), (int)num(3), (int)num(4), (float)num(5), (int)num(6), workspace_of(&ops));
+                         (int)num(2), (int)num(3), (int)num(4), (float)num(5), (int)num(6), workspace_of(&ops), listed ? arg(9) : Tensor(),
+                         listed ? &l : nullptr);
+  } else if (op == "latent_transpose") {
+    ops.latent_transpose(arg(0), arg(1), (int)num(0));
   } else if (op == "moe_experts_gated") {
     // h, ids, wts, gate_up, down, y; experts, kind, limit, alpha
     ops.moe_experts_gated(arg(0), arg(1), arg(2), arg(3), arg(4), arg(5), (int)num(0), (Ops::GatedAct)(int)num(1), (float)num(2),

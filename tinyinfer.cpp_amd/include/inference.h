@@ -366,16 +366,28 @@ class Ops {
   // out [M, 2H] = [a | b] in out's dtype
   void concat_round(const Tensor& a, const Tensor& b, const Tensor& out);
   // Latent attention (a token keeps a normed latent of `rank` numbers and one rotated key part of `rot_dim`, pool
-  // [pages][P][rank + rot_dim]; a head's key is [W_uk c | kr], its value W_uv c).  proj f32 [M, >= off_kv + rank + rot_dim]:
+  // [pages][P][rank + rot_dim], or [pages][P][2 rank + rot_dim]: then a page holds its P rows of rank + rot_dim and behind
+  // them the latents a second time, transposed [rank][P], which the matrix-core kernels read; a head's key is [W_uk c | kr],
+  // its value W_uv c).  proj f32 [M, >= off_kv + rank + rot_dim]:
   // the heads' queries [heads][dim + rot_dim] from column 0, latent and key part from column off_kv.
   // latent_prep: the latent normed (norm_w, eps) and the key part rotated into the token's row; the heads' rotated parts turned in place
   void latent_prep(const Tensor& proj, int off_kv, const Tensor& norm_w, float eps, const Rotation& rot, const int* positions,
                    const int* slots, const CacheView& view, const Tensor& pool, int heads, int dim, int rot_dim, int rank);
   // out [M, heads v_dim] = W_uv (softmax((W_uk^T q | q_rot) . [c | kr] scale; sink) c): scores and softmax in 32-bit, the
   // sink (f32 [heads], may be undefined) in the denominator only; scratch from `ws`
+  // w_uk_t (w_uk's heads transposed, `latent_transpose`) and `lists` (tiles of up to 64 rows of entries of several tokens, the
+  // rows of single tokens; `context`: the longest context of such a row, whose keys several workgroups may share): with both,
+  // bfloat16, pages with the transposed latents and sizes they serve, the matrix-core kernels run
+  struct LatentLists { const int* tiles = nullptr; int n_tiles = 0; const int* rows = nullptr; int n_rows = 0;
+                       const int* entry_meta = nullptr; int context = 0; };
   void latent_attention(const Tensor& proj, const Tensor& w_uk, const Tensor& w_uv, const Tensor& sink, const Tensor& pool,
                         const CacheView& view, const int* positions, const int* slots, const Tensor& out, int heads, int dim,
-                        int rot_dim, int rank, int v_dim, float scale, int window, Workspace& ws);
+                        int rot_dim, int rank, int v_dim, float scale, int window, Workspace& ws, const Tensor& w_uk_t = Tensor(),
+                        const LatentLists* lists = nullptr);
+  // dst [heads][cols][rows] = src [heads rows][cols], every head's matrix transposed
+  void latent_transpose(const Tensor& src, const Tensor& dst, int heads);
+  // whether the matrix-core kernels serve these sizes
+  bool latent_fast(int heads, int dim, int rot_dim, int rank, int v_dim, int page_size);
   // ---- layers that norm what a sublayer returns; short convolutions; differential attention; mixtures of experts
   // x (+)= y / rms(y) * gain (32-bit; gain is the factor itself).  accumulate false: x is overwritten (y may be x).
   // gather (device int32 [M][n_gather]): row m of y is the sum of the rows y[gather[m][k]], k ascending; no list and

@@ -100,7 +100,7 @@ _LIB_OF = {"embed": "core", "rmsnorm": "core", "rope_neox": "core", "rope_table"
            "scale": "residual", "short_conv": "diff_attention", "diff_qk_prep": "diff_attention", "diff_attention": "diff_attention",
            "moe_route": "moe", "moe_experts": "moe", "moe_experts_gated": "moe", "qkv_prep_write": "pointwise", "dyt": "pointwise",
            "gated_act": "pointwise", "concat_round": "pointwise", "latent_prep": "latent_attention",
-           "latent_attention": "latent_attention"}
+           "latent_attention": "latent_attention", "latent_transpose": "latent_attention"}
 
 
 class Ops:
@@ -434,9 +434,24 @@ class Ops:
         self._call("latent_prep", [proj, norm_w, inv_freq, rope_table, positions, slots, table, pool],
                    [off_kv, eps, heads, dim, rot_dim, rank, rot_dims, mag])
 
-    def latent_attention(self, proj, w_uk, w_uv, sink, pool, table, positions, slots, out, heads, dim, rot_dim, rank, v_dim, scale, window=0):
-        self._call("latent_attention", [proj, w_uk, w_uv, sink, pool, table, positions, slots, out],
-                   [heads, dim, rot_dim, rank, v_dim, scale, int(window or 0)])
+    def latent_attention(self, proj, w_uk, w_uv, sink, pool, table, positions, slots, out, heads, dim, rot_dim, rank, v_dim, scale, window=0,
+                         w_uk_t=None, tiles=None, rows=None, entries=None, all_rows=False, context=0):
+        """pool [pages, P, rank + rot_dim], or [pages, P, 2 rank + rot_dim] (a page: its P rows, then the latents transposed
+        [rank][P]).  w_uk_t (`latent_transpose` of w_uk) with tiles int32 [n, 3] = (entry, first row, rows <= 64) and entries
+        int32 [R, 4] = (row0, tokens, start, -), rows int32 [n] (or all_rows: every row is a single token): the bfloat16
+        matrix-core kernels; without them every row is walked on its own."""
+        tensors, numbers = [proj, w_uk, w_uv, sink, pool, table, positions, slots, out], [heads, dim, rot_dim, rank, v_dim, scale, int(window or 0)]
+        libs = ["latent_attention"]
+        if w_uk_t is not None:
+            tensors += [w_uk_t, tiles, rows, entries]
+            numbers += [proj.shape[0] if all_rows else 0, int(context or 0)]
+            if out.dtype == native.torch().bfloat16:
+                libs.append("latent_attention_bf16")
+        self._call("latent_attention", tensors, numbers, libs=libs)
+
+    def latent_transpose(self, src, dst, heads):
+        """dst [heads cols, rows] = src [heads rows, cols], every head's matrix transposed."""
+        self._call("latent_transpose", [src, dst], [heads])
 
     def moe_experts(self, h, ids, wts, up, down, y, experts, scale_input=True):
         """y f32 [M, W] = sum over a token's experts; up [experts F, W], down [experts W, F]."""

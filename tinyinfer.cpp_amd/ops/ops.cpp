@@ -985,8 +985,10 @@ void Ops::concat_round(const Tensor& a, const Tensor& b, const Tensor& out) {
 }
 
 static void check_latent_pool(const char* what, const Tensor& pool, int rank, int rot_dim, DType dt) {
-  require(pool.ndim == 3 && pool.shape[2] == (int64_t)rank + rot_dim && pool.dtype == dt && pool.contiguous(),
-          std::string(what) + ": pool " + pool.describe() + " does not fit [pages, P, " + std::to_string(rank + rot_dim) + "] of " + dtype_name(dt));
+  require(pool.ndim == 3 && (pool.shape[2] == (int64_t)rank + rot_dim || pool.shape[2] == (int64_t)2 * rank + rot_dim) && pool.dtype == dt &&
+              pool.contiguous(),
+          std::string(what) + ": pool " + pool.describe() + " does not fit [pages, P, " + std::to_string(rank + rot_dim) + " (+ " +
+              std::to_string(rank) + ")] of " + dtype_name(dt));
 }
 
 void Ops::latent_prep(const Tensor& proj, int off_kv, const Tensor& norm_w, float eps, const Rotation& rot, const int* positions,
@@ -996,20 +998,36 @@ void Ops::latent_prep(const Tensor& proj, int off_kv, const Tensor& norm_w, floa
               proj.shape[1] >= (int64_t)off_kv + rank + rot_dim,
           "latent_prep: proj " + proj.describe() + " does not hold the queries and the latent");
   require(norm_w.dtype == DType::F32 && norm_w.numel() == rank, "latent_prep: the latent's norm weight " + norm_w.describe() + " does not fit");
-  require(pool.ndim == 3 && pool.shape[2] == (int64_t)rank + rot_dim && pool.contiguous(), "latent_prep: pool " + pool.describe() + " does not fit");
+  require(pool.ndim == 3 && (pool.shape[2] == (int64_t)rank + rot_dim || pool.shape[2] == (int64_t)2 * rank + rot_dim) && pool.contiguous(),
+          "latent_prep: pool " + pool.describe() + " does not fit");
   const int rot_dims = rot.inv_freq ? (rot.dims > 0 ? rot.dims : rot_dim) : 0;
   require(rot_dims % 2 == 0 && rot_dims <= rot_dim, "latent_prep: " + std::to_string(rot_dims) + " rotated entries do not fit " + std::to_string(rot_dim));
   int rc = KERNEL("latent_attention", ti_latent_prep)(code(pool.dtype, "latent_prep"), (float*)proj.data, (int)proj.shape[1], off_kv,
                                                       (const float*)norm_w.data, eps, rot.inv_freq, rot.table, rot.table_len, rot.mag,
                                                       rot_dims, positions, slots, view.table, view.table_width, pool.data,
-                                                      (int)proj.shape[0], heads, dim, rot_dim, rank, (int)pool.shape[1],
-                                                      (hipStream_t)launch_stream());
+                                                      (long)(pool.shape[1] * pool.shape[2]), (int)proj.shape[0], heads, dim, rot_dim,
+                                                      rank, (int)pool.shape[1], (hipStream_t)launch_stream());
   check("latent_attention", rc, "latent_prep");
+}
+
+void Ops::latent_transpose(const Tensor& src, const Tensor& dst, int heads) {
+  require(src.ndim == 2 && dst.ndim == 2 && heads > 0 && src.shape[0] % heads == 0 && dst.shape[0] == (int64_t)heads * src.shape[1] &&
+              dst.shape[1] == src.shape[0] / heads && src.dtype == dst.dtype && src.contiguous() && dst.contiguous(),
+          "latent_transpose: " + src.describe() + " and " + dst.describe() + " do not fit");
+  int rc = KERNEL("latent_attention", ti_latent_transpose)(code(src.dtype, "latent_transpose"), src.data, dst.data, heads,
+                                                           (int)(src.shape[0] / heads), (int)src.shape[1], (hipStream_t)launch_stream());
+  check("latent_attention", rc, "latent_transpose");
+}
+
+bool Ops::latent_fast(int heads, int dim, int rot_dim, int rank, int v_dim, int page_size) {
+  return use.fast_attention && kernel_library_available("latent_attention_bf16") &&
+         KERNEL("latent_attention_bf16", ti_latent_bf16_served)(heads, dim, rot_dim, rank, v_dim, page_size) != 0;
 }
 
 void Ops::latent_attention(const Tensor& proj, const Tensor& w_uk, const Tensor& w_uv, const Tensor& sink, const Tensor& pool,
                            const CacheView& view, const int* positions, const int* slots, const Tensor& out, int heads, int dim,
-                           int rot_dim, int rank, int v_dim, float scale, int window, Workspace& ws) {
+                           int rot_dim, int rank, int v_dim, float scale, int window, Workspace& ws, const Tensor& w_uk_t,
+                           const LatentLists* lists) {
   TIMED("latent_attention " + dims(proj));
   const int64_t M = proj.shape[0];
   require(proj.ndim == 2 && proj.dtype == DType::F32 && proj.contiguous() && proj.shape[1] >= (int64_t)heads * (dim + rot_dim),
@@ -1022,16 +1040,56 @@ void Ops::latent_attention(const Tensor& proj, const Tensor& w_uk, const Tensor&
   require(out.ndim == 2 && out.shape[0] == M && out.shape[1] == (int64_t)heads * v_dim && out.contiguous(), "latent_attention: out has the wrong shape");
   if (M == 0) return;
   const int dt = code(out.dtype, "latent_attention");
+  const long page_elems = (long)(pool.shape[1] * pool.shape[2]);
+  const int P = (int)pool.shape[1];
+  const float* sink_p = sink.defined() ? (const float*)sink.data : nullptr;
+  void* stream = launch_stream();
+  // the matrix cores: bfloat16, pages that hold the latents transposed as well, the heads' W_uk transposed, the step's lists
+  if (lists && out.dtype == DType::BF16 && w_uk_t.defined() && pool.shape[2] == (int64_t)2 * rank + rot_dim &&
+      (lists->n_tiles == 0 || (lists->tiles && lists->entry_meta)) && latent_fast(heads, dim, rot_dim, rank, v_dim, P)) {
+    require(w_uk_t.dtype == DType::BF16 && w_uk_t.contiguous() && w_uk_t.numel() == w_uk.numel(), "latent_attention: w_uk_t " + w_uk_t.describe() + " does not fit");
+    Tensor qa = ws.tensor("latent.qa16", DType::BF16, {M, (int64_t)heads * (rank + rot_dim)});
+    Tensor o = ws.tensor("latent.o16", DType::BF16, {M, (int64_t)heads * rank});
+    int rc = KERNEL("latent_attention_bf16", ti_latent_absorb_bf16)((const float*)proj.data, (int)proj.shape[1], w_uk_t.data, qa.data, (int)M,
+                                                                    heads, dim, rot_dim, rank, (hipStream_t)stream);
+    check("latent_attention_bf16", rc, "latent_attention(absorb, bf16)");
+    if (lists->n_tiles) {
+      rc = KERNEL("latent_attention_bf16", ti_latent_attention_tiles_bf16)(qa.data, pool.data, page_elems, view.table, view.table_width,
+                                                                           lists->tiles, lists->entry_meta, sink_p, o.data, lists->n_tiles,
+                                                                           heads, rank, rot_dim, P, scale, window, (hipStream_t)stream);
+      check("latent_attention_bf16", rc, "latent_attention(tiles, bf16)");
+    }
+    if (lists->n_rows) {
+      // few rows and long contexts: several workgroups share a row's keys, until about one workgroup a compute unit runs
+      const int groups = (heads + 15) / 16;
+      int reach = lists->context;
+      if (window > 0) reach = std::min(reach, window);
+      int splits = 1;
+      if (reach > 0) splits = std::max(1, std::min({16, compute_units() / std::max(1, lists->n_rows * groups), reach / 128}));
+      if (use.force_decode_splits > 0) splits = std::min(64, use.force_decode_splits);
+      float* part = nullptr;
+      if (splits > 1) {
+        const long floats = KERNEL("latent_attention_bf16", ti_latent_attention_rows_scratch)(lists->n_rows, heads, rank, rot_dim, splits);
+        part = (float*)ws.get("latent.part", (size_t)floats * 4);
+      }
+      rc = KERNEL("latent_attention_bf16", ti_latent_attention_rows_bf16)(qa.data, pool.data, page_elems, view.table, view.table_width,
+                                                                          positions, slots, lists->rows, sink_p, o.data, lists->n_rows, heads,
+                                                                          rank, rot_dim, P, scale, window, part, splits, (hipStream_t)stream);
+      check("latent_attention_bf16", rc, "latent_attention(rows, bf16)");
+    }
+    took("[mfma]");
+    rc = KERNEL("latent_attention_bf16", ti_latent_expand_bf16)(o.data, w_uv.data, out.data, (int)M, heads, rank, v_dim, (hipStream_t)stream);
+    check("latent_attention_bf16", rc, "latent_attention(expand, bf16)");
+    return;
+  }
   Tensor qa = ws.tensor("latent.qa", DType::F32, {M, (int64_t)heads * (rank + rot_dim)});
   Tensor o = ws.tensor("latent.o", DType::F32, {M, (int64_t)heads * rank});
-  void* stream = launch_stream();
   int rc = KERNEL("latent_attention", ti_latent_absorb)(dt, (const float*)proj.data, (int)proj.shape[1], w_uk.data, (float*)qa.data, (int)M,
                                                         heads, dim, rot_dim, rank, (hipStream_t)stream);
   check("latent_attention", rc, "latent_attention(absorb)");
-  rc = KERNEL("latent_attention", ti_latent_attention_rows)(dt, (const float*)qa.data, pool.data, view.table, view.table_width, positions,
-                                                            slots, sink.defined() ? (const float*)sink.data : nullptr, (float*)o.data,
-                                                            (int)M, heads, rank, rot_dim, (int)pool.shape[1], scale, window,
-                                                            (hipStream_t)stream);
+  rc = KERNEL("latent_attention", ti_latent_attention_rows)(dt, (const float*)qa.data, pool.data, page_elems, view.table, view.table_width,
+                                                            positions, slots, sink_p, (float*)o.data, (int)M, heads, rank, rot_dim, P, scale,
+                                                            window, (hipStream_t)stream);
   check("latent_attention", rc, "latent_attention(rows)");
   took("[generic]");
   rc = KERNEL("latent_attention", ti_latent_expand)(dt, (const float*)o.data, w_uv.data, out.data, (int)M, heads, rank, v_dim,

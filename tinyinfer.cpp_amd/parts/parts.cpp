@@ -1796,7 +1796,9 @@ class GatedFFN final : public FeedForwardPart {
 // (v_head_dim rows a head); score = (q_plain . k_plain + q_rot . k_rot) scale; causal (`window` optional); the softmax's
 // denominator also holds exp(sink_h), a learned number a head (`sink`, optional).  Then the output projection.
 // Scores, softmax, the latent's norm and the rotation are 32-bit.  Tensor names: prefix + ".q", ".dkv", ".dkv.norm", ".uk",
-// ".uv", ".sink", ".o".
+// ".uv", ".sink", ".o".  Where the sizes allow (a latent of a multiple of 16 up to 512, latent and key part together a
+// multiple of 8 up to 576, an unrotated query size that is a multiple of 8, a value size that is a multiple of 16) a page holds
+// the latents a second time, transposed, and bfloat16 steps run on the matrix cores.
 class LatentAttention final : public MixerPart {
  public:
   LatentAttention(const std::string& prefix, const Json& p, const PartChildren& children) : MixerPart(prefix) {
@@ -1819,6 +1821,8 @@ class LatentAttention final : public MixerPart {
     if (!pos && p.has("pos")) pos = std::dynamic_pointer_cast<PositionPart>(build_part("pos", PartSpec::from_json(p.at("pos")), prefix));
     nq = (int64_t)heads * (dim + rot_dim);
     nkv = (int64_t)rank + rot_dim;
+    // sizes the matrix-core kernels take: the pages then hold the latents a second time, transposed
+    transposed = dim % 8 == 0 && (dim + rot_dim) % 4 == 0 && rank % 16 == 0 && rank <= 512 && nkv % 8 == 0 && nkv <= 576 && v_dim % 16 == 0;
   }
   const char* kind_name() const override { return "latent_attention"; }
   bool can_store() const override { return true; }
@@ -1865,14 +1869,74 @@ class LatentAttention final : public MixerPart {
       if (kv.first == name("sink")) sink = src.fetch(kv.first, kv.second);
       if (kv.first == name("o")) w_o = src.fetch(kv.first, kv.second);
     }
+    if (transposed && w_uk.dtype == DType::BF16) w_uk_t = src.alloc(w_uk.dtype, {(int64_t)heads * rank, (int64_t)dim});
+    uk_transposed = false;
+  }
+  void prepare(Ops& ops, int max_seq) override {
+    (void)max_seq;
+    if (w_uk_t.defined() && !uk_transposed) {
+      ops.latent_transpose(w_uk, w_uk_t, heads);
+      uk_transposed = true;
+    }
   }
   bool has_cache() const override { return true; }
   CacheNeed cache_need() const override {
     CacheNeed n;
     n.kind = CacheNeed::PagedRows;
-    n.row_shape = {nkv};
+    n.row_shape = {transposed ? nkv + rank : nkv};      // a page: its rows of nkv, then (transposed) the latents again as [rank][rows]
     n.window = window;
     return n;
+  }
+  // The lists of the matrix-core kernels: tiles of TILE_ROWS query rows over the entries of several tokens, and the rows
+  // of single-token entries.  Every such mixer of a model asks for the same lists; the first one builds them.
+  static constexpr int TILE_ROWS = 64;
+  void plan(StepPlan& plan) const override {
+    if (!transposed || plan.decode_only() || plan.has("lattn.tiles")) return;
+    const auto& entries = plan.entries();
+    size_t n_tiles = 0, n_rows = 0;
+    for (const auto& e : entries) {
+      if (e.n_tokens > 1) n_tiles += (size_t)(e.n_tokens + TILE_ROWS - 1) / TILE_ROWS;
+      else ++n_rows;
+    }
+    int* tiles = plan.ints("lattn.tiles", 3 * n_tiles);
+    int* rows = plan.ints("lattn.rows", n_rows);
+    struct Tile { int keys, entry, row, n; };
+    std::vector<Tile> order;
+    order.reserve(n_tiles);
+    size_t r = 0;
+    for (size_t i = 0; i < entries.size(); ++i) {
+      const auto& e = entries[i];
+      if (e.n_tokens == 1) {
+        rows[r++] = e.row0;
+        continue;
+      }
+      for (int q0 = 0; q0 < e.n_tokens; q0 += TILE_ROWS) {
+        const int n = std::min(TILE_ROWS, e.n_tokens - q0);
+        order.push_back({e.start + q0 + n, (int)i, e.row0 + q0, n});      // the keys its last row sees
+      }
+    }
+    // from the tile that walks the most keys to the one that walks the fewest: the long ones start first
+    std::stable_sort(order.begin(), order.end(), [](const Tile& a, const Tile& b) { return a.keys > b.keys; });
+    for (size_t t = 0; t < order.size(); ++t) {
+      tiles[3 * t] = order[t].entry;
+      tiles[3 * t + 1] = order[t].row;
+      tiles[3 * t + 2] = order[t].n;
+    }
+  }
+  Ops::LatentLists lists(const StepContext& ctx) const {
+    Ops::LatentLists l;
+    l.entry_meta = ctx.entry_meta;
+    // a captured graph serves every later step of its shape: what it launches is sized for the longest sequence
+    l.context = ctx.plan && ctx.plan->sized_for_longest() ? ctx.plan->max_seq() : ctx.max_context;
+    if (ctx.decode_only) {
+      l.n_rows = (int)ctx.M;
+      return l;
+    }
+    l.tiles = ctx.planned("lattn.tiles");
+    l.n_tiles = (int)(ctx.planned_size("lattn.tiles") / 3);
+    l.rows = ctx.planned("lattn.rows");
+    l.n_rows = (int)ctx.planned_size("lattn.rows");
+    return l;
   }
   void run(StepContext& ctx, const Rows& h, const Tensor& out, Ops::Epilogue epi) {
     const int64_t M = h.t.shape[0];
@@ -1885,21 +1949,25 @@ class LatentAttention final : public MixerPart {
     if (pos && !pos->fused(rot)) throw EngineError("latent_attention: the position encoding '" + std::string(pos->kind_name()) + "' has no fused form");
     ctx.ops.latent_prep(proj, (int)nq, norm_w, eps, rot, ctx.positions, ctx.slots, view, pool, heads, dim, rot_dim, rank);
     Tensor a = ctx.buf("latent.out", ctx.act_dtype, {M, (int64_t)heads * v_dim});
+    const Ops::LatentLists l = lists(ctx);
     ctx.ops.latent_attention(proj, w_uk, w_uv, sink, pool, view, ctx.positions, ctx.slots, a, heads, dim, rot_dim, rank, v_dim, scale,
-                             window, ctx.ws);
+                             window, ctx.ws, w_uk_t, transposed && ctx.plan ? &l : nullptr);
     ctx.ops.linear(a, w_o, out, epi, false);
   }
   void forward(StepContext& ctx, const Rows& h, const Tensor& x) override { run(ctx, h, x, Ops::Add); }
   void forward_store(StepContext& ctx, const Rows& h, const Tensor& y) override { run(ctx, h, y, Ops::Store); }
   std::vector<std::pair<std::string, Tensor>> held() const override {
-    return {{"w_in", w_in}, {"norm_w", norm_w}, {"w_uk", w_uk}, {"w_uv", w_uv}, {"sink", sink}, {"w_o", w_o}};
+    return {{"w_in", w_in}, {"norm_w", norm_w}, {"w_uk", w_uk}, {"w_uv", w_uv}, {"sink", sink}, {"w_o", w_o}, {"w_uk_t", w_uk_t}};
   }
   int64_t hidden = 0, nq = 0, nkv = 0;
   int heads = 0, dim = 0, rot_dim = 0, v_dim = 0, rank = 0, window = 0;
   bool has_sink = true;
+  bool transposed = false;      // the pages hold the latents transposed as well (sizes the matrix-core kernels take)
+  bool uk_transposed = false;   // w_uk_t has been filled
   float eps = 1e-6f, scale = 1.f;
   std::shared_ptr<PositionPart> pos;
   Tensor w_in, norm_w, w_uk, w_uv, sink, w_o;
+  Tensor w_uk_t;                // bfloat16: every head's W_uk transposed, [heads][rank][dim]
 };
 
 // Keeps a copy of the residual as it stands, under `name`, for a later block of the same step (the embedding's output that
