@@ -4,7 +4,7 @@
 // rows: the first product reduces over the R + r entries of a row, the second over the keys, and each reads its operand
 // along the dimension it reduces over, straight from memory.  Every head attends over the same rows with its absorbed
 // query qa = [W_uk^T q_plain | q_rot]; the weighted latent o goes through W_uv afterwards:
-//   latent_absorb_mfma   qa^T (R x 16 tokens)   = W_uk_h^T (R x d) . q_plain^T      one workgroup per (16 tokens, head)
+//   latent_absorb_mfma   qa^T (R x 16 tokens)   = W_uk_h^T (R x d) . q_plain^T      a wavefront per (16 tokens, head, 16 entries)
 //   S^T (16 keys x 16 columns)                   = [c | kr] (16 x DK) . qa^T
 //   O^T (R x 16 columns)                        += c^T (R x 32 keys) . P^T
 //   latent_expand_mfma   out^T (dv x 16 tokens)  = W_uv_h (dv x R) . o^T
@@ -79,21 +79,34 @@ __device__ __forceinline__ void latent_pair(const LatPages& kv, const LFrag8* qf
     rowB = (safe_key % kv.P) & ~15;
   }
   const bool plain = validA && validB && keyA >= lo_max && keyB + 15 <= hi_min;
-  const bf16_t* ka = kv.pool + (size_t)pageA * kv.page_elems + (size_t)(rowA + r16) * kv.DK + quad * 8;
-  const bf16_t* kb = kv.pool + (size_t)pageB * kv.page_elems + (size_t)(rowB + r16) * kv.DK + quad * 8;
+  // Every load is issued whatever the sizes (a step or block beyond them reads the last one that exists and counts as zero),
+  // so that nothing stands between the loads and they are all in flight together.
+  const bf16_t* ka = kv.pool + (size_t)pageA * kv.page_elems + (size_t)(rowA + r16) * kv.DK;
+  const bf16_t* kb = kv.pool + (size_t)pageB * kv.page_elems + (size_t)(rowB + r16) * kv.DK;
+  LFrag8 fa[NKS], fb[NKS];
+#pragma unroll
+  for (int s = 0; s < NKS; ++s) {
+    const int at = min(s * 32 + quad * 8, kv.DK - 8);
+    fa[s].u = *reinterpret_cast<const uint4*>(ka + at);
+    fb[s].u = *reinterpret_cast<const uint4*>(kb + at);
+  }
+  // the transposed latents: row (entry) 16 d + lane % 16, keys 4 (lane / 16) .. + 3 of either block
+  const size_t t_base = (size_t)kv.P * kv.DK;
+  const bf16_t* va = kv.pool + (size_t)pageA * kv.page_elems + t_base + rowA + quad * 4;
+  const bf16_t* vb = kv.pool + (size_t)pageB * kv.page_elems + t_base + rowB + quad * 4;
   floatx4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int s = 0; s < NKS; ++s) {
-    if (s * 32 < kv.DK) {
-      LFrag8 a, b;
-      a.u = b.u = make_uint4(0u, 0u, 0u, 0u);
-      if (s * 32 + quad * 8 < kv.DK) {
-        a.u = *reinterpret_cast<const uint4*>(ka + s * 32);
-        b.u = *reinterpret_cast<const uint4*>(kb + s * 32);
-      }
-      sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qf[s].v, sa, 0, 0, 0);
-      sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b.v, qf[s].v, sb, 0, 0, 0);
-    }
+    if (!(s * 32 + quad * 8 < kv.DK)) fa[s].u = fb[s].u = make_uint4(0u, 0u, 0u, 0u);
+    sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[s].v, qf[s].v, sa, 0, 0, 0);
+    sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[s].v, qf[s].v, sb, 0, 0, 0);
+  }
+  uint2 ta[NRT], tb[NRT];
+#pragma unroll
+  for (int d = 0; d < NRT; ++d) {
+    const int c = min(d * 16 + r16, kv.R - 1);
+    ta[d] = *reinterpret_cast<const uint2*>(va + (size_t)c * kv.P);
+    tb[d] = *reinterpret_cast<const uint2*>(vb + (size_t)c * kv.P);
   }
   float sv[8];
   unsigned keepA[2] = {0xFFFFFFFFu, 0xFFFFFFFFu}, keepB[2] = {0xFFFFFFFFu, 0xFFFFFFFFu};
@@ -136,20 +149,13 @@ __device__ __forceinline__ void latent_pair(const LatPages& kv, const LFrag8* qf
     st.m = m_new;
   }
   st.l += ps;
-  // the transposed latents: row (entry) 16 d + lane % 16, keys 4 (lane / 16) .. + 3 of either block
-  const size_t t_base = (size_t)kv.P * kv.DK;
-  const bf16_t* va = kv.pool + (size_t)pageA * kv.page_elems + t_base + (size_t)r16 * kv.P + rowA + quad * 4;
-  const bf16_t* vb = kv.pool + (size_t)pageB * kv.page_elems + t_base + (size_t)r16 * kv.P + rowB + quad * 4;
-  const unsigned v_step = 16u * kv.P;
 #pragma unroll
   for (int d = 0; d < NRT; ++d) {
-    if (d * 16 < kv.R) {
-      const uint2 a = *reinterpret_cast<const uint2*>(va + d * v_step);
-      const uint2 b = *reinterpret_cast<const uint2*>(vb + d * v_step);
-      LFrag8 v;
-      v.u = make_uint4(a.x & keepA[0], a.y & keepA[1], b.x & keepB[0], b.y & keepB[1]);
-      st.o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v.v, pf.v, st.o[d], 0, 0, 0);
-    }
+    const bool in = d * 16 + r16 < kv.R;      // a row beyond the latent: the output's rows there are never stored
+    LFrag8 v;
+    v.u = make_uint4(ta[d].x & keepA[0], ta[d].y & keepA[1], tb[d].x & keepB[0], tb[d].y & keepB[1]);
+    if (!in) v.u = make_uint4(0u, 0u, 0u, 0u);
+    st.o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v.v, pf.v, st.o[d], 0, 0, 0);
   }
 }
 
@@ -159,8 +165,8 @@ __device__ __forceinline__ void load_query(const bf16_t* qrow, int DK, LFrag8* q
   const int quad = (threadIdx.x & 63) >> 4;
 #pragma unroll
   for (int s = 0; s < NKS; ++s) {
-    qf[s].u = make_uint4(0u, 0u, 0u, 0u);
-    if (s * 32 + quad * 8 < DK) qf[s].u = *reinterpret_cast<const uint4*>(qrow + s * 32 + quad * 8);
+    qf[s].u = *reinterpret_cast<const uint4*>(qrow + min(s * 32 + quad * 8, DK - 8));
+    if (!(s * 32 + quad * 8 < DK)) qf[s].u = make_uint4(0u, 0u, 0u, 0u);
   }
 }
 
@@ -288,26 +294,50 @@ latent_rows_mfma_kernel(const bf16_t* __restrict__ qa, const bf16_t* __restrict_
   store_share<NRT>(st, part + (((size_t)blockIdx.x * gridDim.y + blockIdx.y) * n_splits + blockIdx.z) * (NRT * 4 + 2) * 64, lane);
 }
 
-// one wavefront per (row, 16 heads): the shares of the workgroups that split the row's keys, in ascending order
+// one workgroup per (row, 16 heads): the shares of the workgroups that split the row's keys.  The first wavefront works out
+// every share's weight (the sink joins the maximum and the sum there); then every thread adds its entries up, shares ascending.
 template <int NRT>
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(256)
 latent_rows_merge_kernel(const float* __restrict__ part, const int* __restrict__ rows, const float* __restrict__ sink,
                          bf16_t* __restrict__ o, int H, int R, int n_splits) {
-  const int lane = threadIdx.x, r16 = lane & 15;
+  constexpr int PER = (NRT * 4 + 2) * 64;
+  __shared__ float w_s[64][64];
+  __shared__ float f_s[64];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r16 = lane & 15, quad = lane >> 4;
   const int m = rows ? rows[blockIdx.x] : blockIdx.x;
   const bool live = (int)blockIdx.y * 16 + r16 < H;
   const int h = live ? blockIdx.y * 16 + r16 : 0;
-  LatState<NRT> st;
-  st.clear();
-  for (int s = 0; s < n_splits; ++s)
-    merge_share<NRT>(st, part + (((size_t)blockIdx.x * gridDim.y + blockIdx.y) * n_splits + s) * (NRT * 4 + 2) * 64, lane);
-  finish_column<NRT>(st, sink, h, R, o + ((size_t)m * H + h) * R, live);
+  const float* base = part + ((size_t)blockIdx.x * gridDim.y + blockIdx.y) * n_splits * PER;
+  if (wave == 0) {
+    const float s2 = sink ? sink[h] * LA_LOG2E : -INFINITY;
+    float mm = s2;
+    for (int s = 0; s < n_splits; ++s) mm = fmaxf(mm, base[(size_t)s * PER + NRT * 4 * 64 + lane]);
+    const float m_safe = (mm == -INFINITY) ? 0.f : mm;
+    float l = 0.f;
+    for (int s = 0; s < n_splits; ++s) {
+      const float w = __builtin_amdgcn_exp2f(base[(size_t)s * PER + NRT * 4 * 64 + lane] - m_safe);
+      w_s[s][lane] = w;
+      l = fmaf(base[(size_t)s * PER + (NRT * 4 + 1) * 64 + lane], w, l);
+    }
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    const float lt = l + (sink ? __builtin_amdgcn_exp2f(s2 - m_safe) : 0.f);
+    f_s[lane] = lt > 0.f ? 1.f / lt : 0.f;
+  }
+  __syncthreads();
+  for (int idx = wave; idx < NRT * 4; idx += 4) {
+    const int c = (idx >> 2) * 16 + quad * 4 + (idx & 3);
+    float acc = 0.f;
+    for (int s = 0; s < n_splits; ++s) acc = fmaf(base[(size_t)s * PER + idx * 64 + lane], w_s[s][lane], acc);
+    if (live && c < R) o[((size_t)m * H + h) * R + c] = f2bf(acc * f_s[lane]);
+  }
 }
 
 // ------------------------------------------------------------------------------------------ the absorbed query
 // qa [M][H][DK] bf16: entries c < R: sum_k q[m, h, k] W_uk[h d + k, c], from w_uk_t [H][R][d] (a head's matrix transposed);
-// entries R + j: q_rot[m, h, j].  proj f32 [M, ld] holds the heads' queries [d + r] from column 0.  Grid (tokens / 16, heads);
-// a wavefront takes the blocks of 16 latent entries wave, wave + 4, ...
+// entries R + j: q_rot[m, h, j].  proj f32 [M, ld] holds the heads' queries [d + r] from column 0.  Grid (tokens / 16, heads,
+// R / 64): a wavefront takes one block of 16 latent entries.  A step of the sum beyond d reads the last one and counts as zero.
 __global__ void __launch_bounds__(256)
 latent_absorb_mfma_kernel(const float* __restrict__ proj, int ldp, const bf16_t* __restrict__ w_uk_t, bf16_t* __restrict__ qa, int M,
                           int H, int d, int r, int R) {
@@ -317,33 +347,36 @@ latent_absorb_mfma_kernel(const float* __restrict__ proj, int ldp, const bf16_t*
   const int tok = blockIdx.x * 16 + r16;
   const bool live = tok < M;
   const float* q = proj + (size_t)(live ? tok : M - 1) * ldp + (size_t)h * (d + r);
-  for (int ct = wave; ct * 16 < R; ct += 4) {
-    const bf16_t* w = w_uk_t + ((size_t)h * R + ct * 16 + r16) * d + quad * 8;
+  const int ct = blockIdx.z * 4 + wave;
+  if (ct * 16 < R) {
+    const bf16_t* w = w_uk_t + ((size_t)h * R + ct * 16 + r16) * d;
     floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
     for (int k0 = 0; k0 < d; k0 += 32) {
+      const int at = min(k0 + quad * 8, d - 8);
       LFrag8 a, b;
-      a.u = b.u = make_uint4(0u, 0u, 0u, 0u);
-      if (k0 + quad * 8 < d) {
-        a.u = *reinterpret_cast<const uint4*>(w + k0);
-        const float4 x = *reinterpret_cast<const float4*>(q + k0 + quad * 8), y = *reinterpret_cast<const float4*>(q + k0 + quad * 8 + 4);
-        b.u = make_uint4(pack_bf16x2(x.x, x.y), pack_bf16x2(x.z, x.w), pack_bf16x2(y.x, y.y), pack_bf16x2(y.z, y.w));
-      }
+      a.u = *reinterpret_cast<const uint4*>(w + at);
+      const float4 x = *reinterpret_cast<const float4*>(q + at), y = *reinterpret_cast<const float4*>(q + at + 4);
+      b.u = make_uint4(pack_bf16x2(x.x, x.y), pack_bf16x2(x.z, x.w), pack_bf16x2(y.x, y.y), pack_bf16x2(y.z, y.w));
+      if (!(k0 + quad * 8 < d)) a.u = make_uint4(0u, 0u, 0u, 0u);
       acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc, 0, 0, 0);
     }
     if (live)
       *reinterpret_cast<uint2*>(qa + ((size_t)tok * H + h) * DK + ct * 16 + quad * 4) =
           make_uint2(pack_bf16x2(acc[0], acc[1]), pack_bf16x2(acc[2], acc[3]));
   }
-  const int n = min(16, M - (int)blockIdx.x * 16);
-  for (int e = threadIdx.x; e < n * r; e += 256) {
-    const int t = blockIdx.x * 16 + e / r, j = e % r;
-    qa[((size_t)t * H + h) * DK + R + j] = f2bf(proj[(size_t)t * ldp + (size_t)h * (d + r) + d + j]);
+  if (blockIdx.z == 0) {
+    const int n = min(16, M - (int)blockIdx.x * 16);
+    for (int e = threadIdx.x; e < n * r; e += 256) {
+      const int t = blockIdx.x * 16 + e / r, j = e % r;
+      qa[((size_t)t * H + h) * DK + R + j] = f2bf(proj[(size_t)t * ldp + (size_t)h * (d + r) + d + j]);
+    }
   }
 }
 
 // ------------------------------------------------------------------------------------------ a head's weighted latent to its output
-// out [M][H dv] bf16: out[m, h dv + j] = sum_c o[m, h, c] W_uv[h dv + j, c].  Grid (tokens / 16, heads); a wavefront takes the
-// blocks of 16 outputs wave, wave + 4, ...
+// out [M][H dv] bf16: out[m, h dv + j] = sum_c o[m, h, c] W_uv[h dv + j, c].  Grid (tokens / 16, heads, dv / 64): a wavefront
+// takes one block of 16 outputs.
 __global__ void __launch_bounds__(256)
 latent_expand_mfma_kernel(const bf16_t* __restrict__ o, const bf16_t* __restrict__ w_uv, bf16_t* __restrict__ out, int M, int H, int R,
                           int dv) {
@@ -352,23 +385,23 @@ latent_expand_mfma_kernel(const bf16_t* __restrict__ o, const bf16_t* __restrict
   const int h = blockIdx.y;
   const int tok = blockIdx.x * 16 + r16;
   const bool live = tok < M;
-  const bf16_t* orow = o + ((size_t)(live ? tok : M - 1) * H + h) * R + quad * 8;
-  for (int jt = wave; jt * 16 < dv; jt += 4) {
-    const bf16_t* w = w_uv + ((size_t)h * dv + jt * 16 + r16) * R + quad * 8;
-    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
-    for (int c0 = 0; c0 < R; c0 += 32) {
-      LFrag8 a, b;
-      a.u = b.u = make_uint4(0u, 0u, 0u, 0u);
-      if (c0 + quad * 8 < R) {
-        a.u = *reinterpret_cast<const uint4*>(w + c0);
-        b.u = *reinterpret_cast<const uint4*>(orow + c0);
-      }
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc, 0, 0, 0);
-    }
-    if (live)
-      *reinterpret_cast<uint2*>(out + (size_t)tok * H * dv + (size_t)h * dv + jt * 16 + quad * 4) =
-          make_uint2(pack_bf16x2(acc[0], acc[1]), pack_bf16x2(acc[2], acc[3]));
+  const int jt = blockIdx.z * 4 + wave;
+  if (jt * 16 >= dv) return;
+  const bf16_t* orow = o + ((size_t)(live ? tok : M - 1) * H + h) * R;
+  const bf16_t* w = w_uv + ((size_t)h * dv + jt * 16 + r16) * R;
+  floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+  for (int c0 = 0; c0 < R; c0 += 32) {
+    const int at = min(c0 + quad * 8, R - 8);
+    LFrag8 a, b;
+    a.u = *reinterpret_cast<const uint4*>(w + at);
+    b.u = *reinterpret_cast<const uint4*>(orow + at);
+    if (!(c0 + quad * 8 < R)) a.u = make_uint4(0u, 0u, 0u, 0u);
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc, 0, 0, 0);
   }
+  if (live)
+    *reinterpret_cast<uint2*>(out + (size_t)tok * H * dv + (size_t)h * dv + jt * 16 + quad * 4) =
+        make_uint2(pack_bf16x2(acc[0], acc[1]), pack_bf16x2(acc[2], acc[3]));
 }
 
 // ------------------------------------------------------------------------------------------ host
@@ -398,7 +431,7 @@ extern "C" int ti_latent_absorb_bf16(const float* proj, int ld, const void* w_uk
                  (d + r) % 4 == 0,
              "latent_absorb (bf16): bad sizes heads=%d dim=%d rot=%d rank=%d ld=%d", H, d, r, R, ld);
   if (M == 0) return 0;
-  latent_absorb_mfma_kernel<<<dim3((M + 15) / 16, H), 256, 0, stream>>>(proj, ld, (const bf16_t*)w_uk_t, (bf16_t*)qa, M, H, d, r, R);
+  latent_absorb_mfma_kernel<<<dim3((M + 15) / 16, H, (R + 63) / 64), 256, 0, stream>>>(proj, ld, (const bf16_t*)w_uk_t, (bf16_t*)qa, M, H, d, r, R);
   TI_LAUNCH_CHECK();
   return 0;
 }
@@ -406,7 +439,7 @@ extern "C" int ti_latent_absorb_bf16(const float* proj, int ld, const void* w_uk
 extern "C" int ti_latent_expand_bf16(const void* o, const void* w_uv, void* out, int M, int H, int R, int dv, hipStream_t stream) {
   TI_REQUIRE(H > 0 && H <= 65535 && R > 0 && R % 8 == 0 && dv > 0 && dv % 16 == 0, "latent_expand (bf16): bad sizes heads=%d rank=%d vdim=%d", H, R, dv);
   if (M == 0) return 0;
-  latent_expand_mfma_kernel<<<dim3((M + 15) / 16, H), 256, 0, stream>>>((const bf16_t*)o, (const bf16_t*)w_uv, (bf16_t*)out, M, H, R, dv);
+  latent_expand_mfma_kernel<<<dim3((M + 15) / 16, H, (dv + 63) / 64), 256, 0, stream>>>((const bf16_t*)o, (const bf16_t*)w_uv, (bf16_t*)out, M, H, R, dv);
   TI_LAUNCH_CHECK();
   return 0;
 }
@@ -454,7 +487,7 @@ extern "C" int ti_latent_attention_rows_bf16(const void* qa, const void* pool, l
   TI_LAUNCH_CHECK();
   if (n_splits > 1) {
     const dim3 mgrid(n_rows, groups);
-#define LA_MERGE(K, V) latent_rows_merge_kernel<V><<<mgrid, 64, 0, stream>>>(part, rows, sink, (bf16_t*)o, H, R, n_splits)
+#define LA_MERGE(K, V) latent_rows_merge_kernel<V><<<mgrid, 256, 0, stream>>>(part, rows, sink, (bf16_t*)o, H, R, n_splits)
     LA_DISPATCH(LA_MERGE);
 #undef LA_MERGE
     TI_LAUNCH_CHECK();
