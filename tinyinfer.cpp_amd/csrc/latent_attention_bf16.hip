@@ -30,8 +30,15 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
 #define LA_LOG2E 1.4426950408889634f
 
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) const u32x4 lds_u32x4;      // reads and writes that are known to go to LDS
+typedef __attribute__((address_space(3))) u32x4 lds_w_u32x4;
+typedef __attribute__((address_space(3))) u32x2 lds_w_u32x2;
+
 union LFrag8 {
   uint4 u;
+  u32x4 n;
   bf16x8 v;
 };
 
@@ -54,15 +61,30 @@ struct LatState {
   }
 };
 
-// One pair of blocks of 16 keys, [keyA, keyA + 16) and [keyA + 16, keyA + 32), for this wavefront's 16 columns.
+// A pair of blocks in LDS, fetched once by a workgroup for its four wavefronts: the 32 key rows, padded by 16 bytes so that
+// the fragments' reads spread over the banks, then the latents transposed: a row per entry that holds, quarter by quarter,
+// four keys of the first block and the same four of the second: a lane's fragment in one read.
+template <int NKS, int NRT>
+struct LatStage {
+  static constexpr int KROW = NKS * 32 + 8;
+  static constexpr int VROW = 32 + 8;
+  static constexpr int K_ELEMS = 32 * KROW;
+  static constexpr int ELEMS = K_ELEMS + NRT * 16 * VROW;
+  static constexpr int K_PIECES = 32 * NKS * 4;            // pieces of 16 bytes: 32 rows of NKS 4
+  static constexpr int V_PIECES = NRT * 16 * 4;            // an entry's 8 keys of either half of either block
+  static constexpr int NK = (K_PIECES + 255) / 256, NV = (V_PIECES + 255) / 256;
+};
+
+// One pair of blocks of 16 keys, [keyA, keyA + 16) and [keyA + 16, keyA + 32), for this wavefront's 16 columns.  `stage`:
+// the pair as a workgroup left it in LDS (null: every wavefront reads its fragments from memory).
 //   qf        qa^T fragments: column lane % 16, entries 32 s + 8 (lane / 16) .. + 7
 //   lo, hi    the keys this lane's column sees: lo <= key <= hi (lo > hi: none)
 //   lo_max, hi_min   the largest lo and the smallest hi of the wavefront's live columns
 //   kv_last   last position of the request that has been written (rows after it hold anything, NaN included)
 //   safe_key  a key whose page exists: loads of blocks that do not count go there, so that they never leave the pool
-template <int NKS, int NRT>
+template <int NKS, int NRT, bool FROM_LDS>
 __device__ __forceinline__ void latent_pair(const LatPages& kv, const LFrag8* qf, int keyA, int lo, int hi, int lo_max, int hi_min,
-                                            int kv_last, int safe_key, float scale2, LatState<NRT>& st) {
+                                            int kv_last, int safe_key, float scale2, LatState<NRT>& st, const bf16_t* stage = nullptr) {
   const int lane = threadIdx.x & 63;
   const int r16 = lane & 15, quad = lane >> 4;
   const int keyB = keyA + 16;
@@ -83,30 +105,43 @@ __device__ __forceinline__ void latent_pair(const LatPages& kv, const LFrag8* qf
   // so that nothing stands between the loads and they are all in flight together.
   const bf16_t* ka = kv.pool + (size_t)pageA * kv.page_elems + (size_t)(rowA + r16) * kv.DK;
   const bf16_t* kb = kv.pool + (size_t)pageB * kv.page_elems + (size_t)(rowB + r16) * kv.DK;
-  LFrag8 fa[NKS], fb[NKS];
-#pragma unroll
-  for (int s = 0; s < NKS; ++s) {
-    const int at = min(s * 32 + quad * 8, kv.DK - 8);
-    fa[s].u = *reinterpret_cast<const uint4*>(ka + at);
-    fb[s].u = *reinterpret_cast<const uint4*>(kb + at);
-  }
   // the transposed latents: row (entry) 16 d + lane % 16, keys 4 (lane / 16) .. + 3 of either block
   const size_t t_base = (size_t)kv.P * kv.DK;
   const bf16_t* va = kv.pool + (size_t)pageA * kv.page_elems + t_base + rowA + quad * 4;
   const bf16_t* vb = kv.pool + (size_t)pageB * kv.page_elems + t_base + rowB + quad * 4;
   floatx4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-  for (int s = 0; s < NKS; ++s) {
-    if (!(s * 32 + quad * 8 < kv.DK)) fa[s].u = fb[s].u = make_uint4(0u, 0u, 0u, 0u);
-    sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[s].v, qf[s].v, sa, 0, 0, 0);
-    sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[s].v, qf[s].v, sb, 0, 0, 0);
-  }
   uint2 ta[NRT], tb[NRT];
+  if (FROM_LDS) {      // LDS answers fast: a fragment is read where it is used
+    using S = LatStage<NKS, NRT>;
 #pragma unroll
-  for (int d = 0; d < NRT; ++d) {
-    const int c = min(d * 16 + r16, kv.R - 1);
-    ta[d] = *reinterpret_cast<const uint2*>(va + (size_t)c * kv.P);
-    tb[d] = *reinterpret_cast<const uint2*>(vb + (size_t)c * kv.P);
+    for (int s = 0; s < NKS; ++s) {
+      LFrag8 a, b;
+      a.n = *(lds_u32x4*)(size_t)(stage + r16 * S::KROW + s * 32 + quad * 8);
+      b.n = *(lds_u32x4*)(size_t)(stage + (16 + r16) * S::KROW + s * 32 + quad * 8);
+      if (!(s * 32 + quad * 8 < kv.DK)) a.u = b.u = make_uint4(0u, 0u, 0u, 0u);
+      sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qf[s].v, sa, 0, 0, 0);
+      sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b.v, qf[s].v, sb, 0, 0, 0);
+    }
+  } else {
+    LFrag8 fa[NKS], fb[NKS];
+#pragma unroll
+    for (int s = 0; s < NKS; ++s) {
+      const int at = min(s * 32 + quad * 8, kv.DK - 8);
+      fa[s].u = *reinterpret_cast<const uint4*>(ka + at);
+      fb[s].u = *reinterpret_cast<const uint4*>(kb + at);
+    }
+#pragma unroll
+    for (int s = 0; s < NKS; ++s) {
+      if (!(s * 32 + quad * 8 < kv.DK)) fa[s].u = fb[s].u = make_uint4(0u, 0u, 0u, 0u);
+      sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[s].v, qf[s].v, sa, 0, 0, 0);
+      sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[s].v, qf[s].v, sb, 0, 0, 0);
+    }
+#pragma unroll
+    for (int d = 0; d < NRT; ++d) {
+      const int c = min(d * 16 + r16, kv.R - 1);
+      ta[d] = *reinterpret_cast<const uint2*>(va + (size_t)c * kv.P);
+      tb[d] = *reinterpret_cast<const uint2*>(vb + (size_t)c * kv.P);
+    }
   }
   float sv[8];
   unsigned keepA[2] = {0xFFFFFFFFu, 0xFFFFFFFFu}, keepB[2] = {0xFFFFFFFFu, 0xFFFFFFFFu};
@@ -152,6 +187,11 @@ __device__ __forceinline__ void latent_pair(const LatPages& kv, const LFrag8* qf
 #pragma unroll
   for (int d = 0; d < NRT; ++d) {
     const bool in = d * 16 + r16 < kv.R;      // a row beyond the latent: the output's rows there are never stored
+    if (FROM_LDS) {
+      const u32x4 t = *(lds_u32x4*)(size_t)(stage + LatStage<NKS, NRT>::K_ELEMS + (d * 16 + r16) * LatStage<NKS, NRT>::VROW + quad * 8);
+      ta[d] = make_uint2(t[0], t[1]);
+      tb[d] = make_uint2(t[2], t[3]);
+    }
     LFrag8 v;
     v.u = make_uint4(ta[d].x & keepA[0], ta[d].y & keepA[1], tb[d].x & keepB[0], tb[d].y & keepB[1]);
     if (!in) v.u = make_uint4(0u, 0u, 0u, 0u);
@@ -226,7 +266,118 @@ latent_tiles_kernel(const bf16_t* __restrict__ qa, const bf16_t* __restrict__ po
   LatState<NRT> st;
   st.clear();
   for (int pr = lo_min / 32; pr <= hi_max / 32; ++pr)
-    latent_pair<NKS, NRT>(kv, qf, pr * 32, lo, hi, lo_max, hi_min, kv_last, hi_max, scale2, st);
+    latent_pair<NKS, NRT, false>(kv, qf, pr * 32, lo, hi, lo_max, hi_min, kv_last, hi_max, scale2, st);
+  finish_column<NRT>(st, sink, h, R, o + ((size_t)row * H + h) * R, live);
+}
+
+// ------------------------------------------------------------------------------------------ tiles, the pairs through LDS
+// The same tiles with the four wavefronts sharing what they read: a pair of blocks is fetched once by the workgroup into one
+// of two LDS stages (through registers: thread t the 16-byte pieces t, t + 256, ...) while the pair before it is multiplied
+// from the other; one barrier a pair.
+template <int NKS, int NRT>
+__device__ __forceinline__ void fetch_pair(const LatPages& kv, int keyA, int kv_last, int safe_key, u32x4* __restrict__ fk, u32x4* __restrict__ fv) {
+  using S = LatStage<NKS, NRT>;
+  const int keyB = keyA + 16;
+  int pageA = keyA <= kv_last ? kv.table[keyA / kv.P] : -1;
+  int pageB = keyB <= kv_last ? kv.table[keyB / kv.P] : -1;
+  int rowA = keyA % kv.P, rowB = keyB % kv.P;
+  if (pageA < 0) {
+    pageA = kv.table[safe_key / kv.P];
+    rowA = (safe_key % kv.P) & ~15;
+  }
+  if (pageB < 0) {
+    pageB = kv.table[safe_key / kv.P];
+    rowB = (safe_key % kv.P) & ~15;
+  }
+  const bf16_t* pa = kv.pool + (size_t)pageA * kv.page_elems;
+  const bf16_t* pb = kv.pool + (size_t)pageB * kv.page_elems;
+#pragma unroll
+  for (int j = 0; j < S::NK; ++j) {
+    const int idx = min((int)threadIdx.x + 256 * j, S::K_PIECES - 1);
+    const int row = idx / (NKS * 4), pc = idx % (NKS * 4);
+    const bf16_t* src = (row < 16 ? pa + (size_t)(rowA + row) * kv.DK : pb + (size_t)(rowB + row - 16) * kv.DK) + min(pc * 8, kv.DK - 8);
+    fk[j] = *reinterpret_cast<const u32x4*>(src);
+  }
+  const size_t t_base = (size_t)kv.P * kv.DK;
+#pragma unroll
+  for (int j = 0; j < S::NV; ++j) {
+    const int idx = min((int)threadIdx.x + 256 * j, S::V_PIECES - 1);
+    const int c = min(idx >> 2, kv.R - 1), blk = (idx >> 1) & 1, half = idx & 1;
+    const bf16_t* src = (blk ? pb + rowB : pa + rowA) + t_base + (size_t)c * kv.P + half * 8;
+    fv[j] = *reinterpret_cast<const u32x4*>(src);
+  }
+}
+
+template <int NKS, int NRT>
+__device__ __forceinline__ void stash_pair(bf16_t* stage, const u32x4* __restrict__ fk, const u32x4* __restrict__ fv) {
+  using S = LatStage<NKS, NRT>;
+#pragma unroll
+  for (int j = 0; j < S::NK; ++j) {
+    const int idx = threadIdx.x + 256 * j;
+    if (idx < S::K_PIECES) *(lds_w_u32x4*)(size_t)(stage + (idx / (NKS * 4)) * S::KROW + (idx % (NKS * 4)) * 8) = fk[j];
+  }
+#pragma unroll
+  for (int j = 0; j < S::NV; ++j) {
+    const int idx = threadIdx.x + 256 * j;
+    if (idx < S::V_PIECES) {
+      const int c = idx >> 2, blk = (idx >> 1) & 1, half = idx & 1;
+      bf16_t* dst = stage + S::K_ELEMS + c * S::VROW + blk * 4;      // keys 8 half .. + 7: the quarters 2 half and 2 half + 1
+      *(lds_w_u32x2*)(size_t)(dst + (2 * half) * 8) = u32x2{fv[j][0], fv[j][1]};
+      *(lds_w_u32x2*)(size_t)(dst + (2 * half + 1) * 8) = u32x2{fv[j][2], fv[j][3]};
+    }
+  }
+}
+
+template <int NKS, int NRT>
+__global__ void __launch_bounds__(256)
+latent_tiles_lds_kernel(const bf16_t* __restrict__ qa, const bf16_t* __restrict__ pool, const int* __restrict__ table, int table_stride,
+                        const int* __restrict__ tiles, const int* __restrict__ entries, const float* __restrict__ sink,
+                        bf16_t* __restrict__ o, int H, int R, int DK, int P, size_t page_elems, float scale2, int window) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  bf16_t* stages = reinterpret_cast<bf16_t*>(lds_raw);
+  using S = LatStage<NKS, NRT>;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r16 = lane & 15;
+  const int e = tiles[3 * blockIdx.x], tile_row0 = tiles[3 * blockIdx.x + 1], tile_n = tiles[3 * blockIdx.x + 2];
+  const int row0 = tile_row0 + 16 * wave, n_rows = tile_n - 16 * wave;      // a wavefront without rows still fetches and waits
+  const int h = blockIdx.y;
+  const int e_row0 = entries[4 * e], e_n = entries[4 * e + 1], e_start = entries[4 * e + 2];
+  const int kv_last = e_start + e_n - 1;
+  const bool live = r16 < n_rows;
+  const int row = live ? row0 + r16 : tile_row0;
+  const int p = e_start + (row - e_row0);
+  const int lo_p = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  const int lo = live ? lo_p : 1, hi = live ? p : 0;
+  int lo_min = live ? lo : 0x7fffffff, lo_max = live ? lo : 0, hi_min = live ? hi : 0x7fffffff, hi_max = live ? hi : -1;
+#pragma unroll
+  for (int x = 1; x < 16; x <<= 1) {
+    lo_min = min(lo_min, __shfl_xor(lo_min, x, 64));
+    lo_max = max(lo_max, __shfl_xor(lo_max, x, 64));
+    hi_min = min(hi_min, __shfl_xor(hi_min, x, 64));
+    hi_max = max(hi_max, __shfl_xor(hi_max, x, 64));
+  }
+  // the workgroup's keys: from the first one its first row sees to its last row's own
+  const int p_first = e_start + (tile_row0 - e_row0), p_last = p_first + tile_n - 1;
+  const int first = ((window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0) / 32, last = p_last / 32;
+  LatPages kv{pool, table + (size_t)e * table_stride, P, DK, R, page_elems};
+  LFrag8 qf[NKS];
+  load_query<NKS>(qa + ((size_t)row * H + h) * DK, DK, qf);
+  LatState<NRT> st;
+  st.clear();
+  u32x4 fk[S::NK], fv[S::NV];
+  fetch_pair<NKS, NRT>(kv, first * 32, kv_last, p_last, fk, fv);
+  stash_pair<NKS, NRT>(stages, fk, fv);
+  __syncthreads();
+  for (int pr = first; pr <= last; ++pr) {
+    const bf16_t* cur = stages + ((pr - first) & 1) * S::ELEMS;
+    bf16_t* nxt = stages + ((pr - first + 1) & 1) * S::ELEMS;
+    // (behind the last pair the same pair is fetched and stashed once more, into the stage nobody reads any longer)
+    fetch_pair<NKS, NRT>(kv, min(pr + 1, last) * 32, kv_last, p_last, fk, fv);
+    if (pr * 32 <= hi_max && pr * 32 + 31 >= lo_min)
+      latent_pair<NKS, NRT, true>(kv, qf, pr * 32, lo, hi, lo_max, hi_min, kv_last, p_last, scale2, st, cur);
+    stash_pair<NKS, NRT>(nxt, fk, fv);
+    __syncthreads();
+  }
   finish_column<NRT>(st, sink, h, R, o + ((size_t)row * H + h) * R, live);
 }
 
@@ -279,7 +430,7 @@ latent_rows_mfma_kernel(const bf16_t* __restrict__ qa, const bf16_t* __restrict_
   LatState<NRT> st;
   st.clear();
   for (int pr = lo_all / 32 + 4 * blockIdx.z + wave; pr <= p / 32; pr += 4 * n_splits)
-    latent_pair<NKS, NRT>(kv, qf, pr * 32, lo, hi, lo_all, p, p, p, scale2, st);
+    latent_pair<NKS, NRT, false>(kv, qf, pr * 32, lo, hi, lo_all, p, p, p, scale2, st);
   for (int w = 1; w < 4; ++w) {
     if (wave == w) store_share<NRT>(st, lds, lane);
     __syncthreads();
@@ -447,7 +598,7 @@ extern "C" int ti_latent_expand_bf16(const void* o, const void* w_uv, void* out,
 // pool bf16 [pages][P rows of R + r | R rows of P]: page_elems elements a page
 extern "C" int ti_latent_attention_tiles_bf16(const void* qa, const void* pool, long page_elems, const int* table, int table_stride,
                                               const int* tiles, const int* entries, const float* sink, void* o, int n_tiles, int H,
-                                              int R, int r, int page_size, float scale, int window, hipStream_t stream) {
+                                              int R, int r, int page_size, float scale, int window, int use_lds, hipStream_t stream) {
   const int DK = R + r;
   TI_REQUIRE(ti_latent_bf16_served(H, 8, 0, R, 16, page_size) && (R + r) % 8 == 0 && R + r <= 576 && H <= 65535 && table_stride > 0 && window >= 0 &&
                  page_elems >= (long)page_size * (DK + R),
@@ -455,9 +606,27 @@ extern "C" int ti_latent_attention_tiles_bf16(const void* qa, const void* pool, 
              page_size, page_elems);
   if (n_tiles == 0) return 0;
   const dim3 grid(n_tiles, H);
-#define LA_TILES(K, V)                                                                                                          \
-  latent_tiles_kernel<K, V><<<grid, 256, 0, stream>>>((const bf16_t*)qa, (const bf16_t*)pool, table, table_stride, tiles, entries, \
-                                                      sink, (bf16_t*)o, H, R, DK, page_size, (size_t)page_elems, scale * LA_LOG2E, window)
+  // keys and latents shared through LDS (use_lds 0: every wavefront fetches its own, for tests and measurements); the two
+  // stages of the largest sizes need more than the 64 KB a kernel may use without asking
+#define LA_TILES(K, V)                                                                                                              \
+  do {                                                                                                                              \
+    if (use_lds) {                                                                                                                  \
+      const int bytes = 2 * LatStage<K, V>::ELEMS * 2;                                                                              \
+      static bool asked = false;                                                                                                    \
+      if (!asked && bytes > 64 * 1024) {                                                                                            \
+        TI_REQUIRE(hipFuncSetAttribute((const void*)latent_tiles_lds_kernel<K, V>, hipFuncAttributeMaxDynamicSharedMemorySize,      \
+                                       bytes) == hipSuccess, "latent_attention (tiles): %d bytes of LDS are refused", bytes);       \
+        asked = true;                                                                                                               \
+      }                                                                                                                             \
+      latent_tiles_lds_kernel<K, V><<<grid, 256, bytes, stream>>>((const bf16_t*)qa, (const bf16_t*)pool, table, table_stride,      \
+                                                                  tiles, entries, sink, (bf16_t*)o, H, R, DK, page_size,           \
+                                                                  (size_t)page_elems, scale * LA_LOG2E, window);                    \
+    } else {                                                                                                                        \
+      latent_tiles_kernel<K, V><<<grid, 256, 0, stream>>>((const bf16_t*)qa, (const bf16_t*)pool, table, table_stride, tiles,       \
+                                                          entries, sink, (bf16_t*)o, H, R, DK, page_size, (size_t)page_elems,       \
+                                                          scale * LA_LOG2E, window);                                                \
+    }                                                                                                                               \
+  } while (0)
   LA_DISPATCH(LA_TILES);
 #undef LA_TILES
   TI_LAUNCH_CHECK();

@@ -160,10 +160,10 @@ int ti_latent_bf16_served(int H, int d, int r, int R, int dv, int page_size);
 // qa bf16 [M, H, R + r] from w_uk_t bf16 [H][R][d] (ti_latent_transpose of w_uk)
 int ti_latent_absorb_bf16(const float* proj, int ld, const void* w_uk_t, void* qa, int M, int H, int d, int r, int R, hipStream_t stream);
 // o bf16 [M, H, R] for the tiles int32 [n][3] = (entry, first row, rows <= 64) of entries int32 [.][4] = (row0, tokens, start, -);
-// the block table's row of a tile is its entry's
+// the block table's row of a tile is its entry's.  use_lds: a tile's four wavefronts share every pair of key blocks through LDS
 int ti_latent_attention_tiles_bf16(const void* qa, const void* pool, long page_elems, const int* table, int table_stride,
                                    const int* tiles, const int* entries, const float* sink, void* o, int n_tiles, int H, int R, int r,
-                                   int page_size, float scale, int window, hipStream_t stream);
+                                   int page_size, float scale, int window, int use_lds, hipStream_t stream);
 // ... and for single rows (rows int32 [n], null: every row): 16 heads a wavefront; n_splits workgroups share a row's keys
 // (part: ti_latent_attention_rows_scratch floats)
 int ti_latent_attention_rows_bf16(const void* qa, const void* pool, long page_elems, const int* table, int table_stride, const int* pos,

@@ -1056,7 +1056,8 @@ void Ops::latent_attention(const Tensor& proj, const Tensor& w_uk, const Tensor&
     if (lists->n_tiles) {
       rc = KERNEL("latent_attention_bf16", ti_latent_attention_tiles_bf16)(qa.data, pool.data, page_elems, view.table, view.table_width,
                                                                            lists->tiles, lists->entry_meta, sink_p, o.data, lists->n_tiles,
-                                                                           heads, rank, rot_dim, P, scale, window, (hipStream_t)stream);
+                                                                           heads, rank, rot_dim, P, scale, window, use.shared_tiles ? 1 : 0,
+                                                                           (hipStream_t)stream);
       check("latent_attention_bf16", rc, "latent_attention(tiles, bf16)");
     }
     if (lists->n_rows) {
