@@ -53,9 +53,9 @@ CONFIGS = {
                 layers=[latent(1, 2, 6, 7, 9, 0.4, 50.0, yarn(8.0, 16, 4.0, 0.5), mlp=moe(1, 1, 9, 3.0, 5, 0.5)),
                         attention(5, 5, 6, 10, 0.5, 1000, 0, 10000.0, mlp=None),
                         attention(2, 2, 10, 7, 0.3, 7, 10, 20.0, mlp=moe(7, 4, 21, 0.8))]),
-    # no loop; widths the matrix-core kernels serve: keys and values of 64 under a window of 50, pages of 16, experts of 32 n
+    # no loop; widths the matrix-core kernels serve: keys and values of 64 under a window of 50, pages of 16, experts of 96
     "wide": dict(architecture="Nazorax", width=128, vocab=320, norm=dict(eps=1e-6),
-                 layers=[attention(4, 2, 64, 64, 0.125, 50, 32, 20000.0, mlp=moe(8, 2, 64, 1.5, 96, 1.0)),
+                 layers=[attention(4, 2, 64, 64, 0.125, 50, 32, 30000.0, mlp=moe(8, 2, 96, 1.5, 160, 1.0)),
                          latent(4, 32, 16, 32, 64, 0.15, 10000.0, yarn(3.0, 64, 16.0, 1.0), mlp=dense(160)),
                          attention(2, 1, 32, 32, 0.18, 0, 32, 10000.0, mlp=moe(6, 1, 32, 2.0))]),
 }

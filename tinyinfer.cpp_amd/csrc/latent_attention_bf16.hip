@@ -445,44 +445,38 @@ latent_rows_mfma_kernel(const bf16_t* __restrict__ qa, const bf16_t* __restrict_
   store_share<NRT>(st, part + (((size_t)blockIdx.x * gridDim.y + blockIdx.y) * n_splits + blockIdx.z) * (NRT * 4 + 2) * 64, lane);
 }
 
-// one workgroup per (row, 16 heads): the shares of the workgroups that split the row's keys.  The first wavefront works out
-// every share's weight (the sink joins the maximum and the sum there); then every thread adds its entries up, shares ascending.
+// The shares of the workgroups that split a row's keys, added up.  Grid (rows, groups of 16 heads, NRT): a wavefront owns one
+// entry of every column's four (its lanes as the shares lie in memory), works out every share's weight itself (the sink joins
+// the maximum and the sum there) and adds its entries up, shares ascending.
 template <int NRT>
 __global__ void __launch_bounds__(256)
 latent_rows_merge_kernel(const float* __restrict__ part, const int* __restrict__ rows, const float* __restrict__ sink,
                          bf16_t* __restrict__ o, int H, int R, int n_splits) {
   constexpr int PER = (NRT * 4 + 2) * 64;
-  __shared__ float w_s[64][64];
-  __shared__ float f_s[64];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r16 = lane & 15, quad = lane >> 4;
   const int m = rows ? rows[blockIdx.x] : blockIdx.x;
   const bool live = (int)blockIdx.y * 16 + r16 < H;
   const int h = live ? blockIdx.y * 16 + r16 : 0;
-  const float* base = part + ((size_t)blockIdx.x * gridDim.y + blockIdx.y) * n_splits * PER;
-  if (wave == 0) {
-    const float s2 = sink ? sink[h] * LA_LOG2E : -INFINITY;
-    float mm = s2;
-    for (int s = 0; s < n_splits; ++s) mm = fmaxf(mm, base[(size_t)s * PER + NRT * 4 * 64 + lane]);
-    const float m_safe = (mm == -INFINITY) ? 0.f : mm;
-    float l = 0.f;
-    for (int s = 0; s < n_splits; ++s) {
-      const float w = __builtin_amdgcn_exp2f(base[(size_t)s * PER + NRT * 4 * 64 + lane] - m_safe);
-      w_s[s][lane] = w;
-      l = fmaf(base[(size_t)s * PER + (NRT * 4 + 1) * 64 + lane], w, l);
-    }
-    l += __shfl_xor(l, 16, 64);
-    l += __shfl_xor(l, 32, 64);
-    const float lt = l + (sink ? __builtin_amdgcn_exp2f(s2 - m_safe) : 0.f);
-    f_s[lane] = lt > 0.f ? 1.f / lt : 0.f;
+  const int idx = blockIdx.z * 4 + wave;
+  const float* base = part + ((size_t)blockIdx.x * gridDim.y + blockIdx.y) * n_splits * PER + lane;
+  const float s2 = sink ? sink[h] * LA_LOG2E : -INFINITY;
+  float mm = s2;
+#pragma unroll 8
+  for (int s = 0; s < n_splits; ++s) mm = fmaxf(mm, base[(size_t)s * PER + NRT * 4 * 64]);
+  const float m_safe = (mm == -INFINITY) ? 0.f : mm;
+  float l = 0.f, acc = 0.f;
+#pragma unroll 8
+  for (int s = 0; s < n_splits; ++s) {
+    const float w = __builtin_amdgcn_exp2f(base[(size_t)s * PER + NRT * 4 * 64] - m_safe);
+    l = fmaf(base[(size_t)s * PER + (NRT * 4 + 1) * 64], w, l);
+    acc = fmaf(base[(size_t)s * PER + idx * 64], w, acc);
   }
-  __syncthreads();
-  for (int idx = wave; idx < NRT * 4; idx += 4) {
-    const int c = (idx >> 2) * 16 + quad * 4 + (idx & 3);
-    float acc = 0.f;
-    for (int s = 0; s < n_splits; ++s) acc = fmaf(base[(size_t)s * PER + idx * 64 + lane], w_s[s][lane], acc);
-    if (live && c < R) o[((size_t)m * H + h) * R + c] = f2bf(acc * f_s[lane]);
-  }
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  const float lt = l + (sink ? __builtin_amdgcn_exp2f(s2 - m_safe) : 0.f);
+  const int c = (idx >> 2) * 16 + quad * 4 + (idx & 3);
+  if (live && c < R) o[((size_t)m * H + h) * R + c] = f2bf(lt > 0.f ? acc / lt : 0.f);
 }
 
 // ------------------------------------------------------------------------------------------ the absorbed query
@@ -655,8 +649,7 @@ extern "C" int ti_latent_attention_rows_bf16(const void* qa, const void* pool, l
 #undef LA_ROWS
   TI_LAUNCH_CHECK();
   if (n_splits > 1) {
-    const dim3 mgrid(n_rows, groups);
-#define LA_MERGE(K, V) latent_rows_merge_kernel<V><<<mgrid, 256, 0, stream>>>(part, rows, sink, (bf16_t*)o, H, R, n_splits)
+#define LA_MERGE(K, V) latent_rows_merge_kernel<V><<<dim3(n_rows, groups, V), 256, 0, stream>>>(part, rows, sink, (bf16_t*)o, H, R, n_splits)
     LA_DISPATCH(LA_MERGE);
 #undef LA_MERGE
     TI_LAUNCH_CHECK();

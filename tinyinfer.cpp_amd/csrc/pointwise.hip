@@ -265,10 +265,12 @@ __global__ void qkv_prep_write_kernel(const float* __restrict__ qkv, const float
   const int r = p % P;
   T* base = pool + (size_t)max(page, 0) * ((size_t)n_kv * P * (dk + dv));
   const int half = inv_freq ? rot_dims / 2 : 0;
-  // queries and keys: a thread takes entry d of a head, and with it entry d + half where d is turned
-  for (int e = threadIdx.x; e < nq + nk; e += blockDim.x) {
+  // queries and keys: a thread takes entry d of a head, and with it entry d + half where d is turned (grid (token, pieces of
+  // 256 entries): a decoded token's few thousand entries spread over workgroups)
+  const int e = blockIdx.y * blockDim.x + threadIdx.x;
+  if (e < nq + nk) {
     const int d = e % dk;
-    if (d >= half && d < 2 * half) continue;      // written by the thread of its partner
+    if (d >= half && d < 2 * half) return;      // written by the thread of its partner
     const bool is_q = e < nq;
     float u = row[e] + (bias ? bias[e] : 0.f);
     float w = 0.f;
@@ -290,11 +292,11 @@ __global__ void qkv_prep_write_kernel(const float* __restrict__ qkv, const float
       if (d < half) st<T>(dst + half, w);
     }
   }
-  if (page < 0) return;
-  T* vbase = base + (size_t)n_kv * P * dk;
-  for (int e = threadIdx.x; e < nv; e += blockDim.x) {
-    const int h = e / dv, d = e % dv;
-    st<T>(vbase + ((size_t)h * dv + d) * P + r, row[nq + nk + e] + (bias ? bias[nq + nk + e] : 0.f));
+  else if (e < nq + nk + nv && page >= 0) {
+    T* vbase = base + (size_t)n_kv * P * dk;
+    const int ev = e - nq - nk;
+    const int h = ev / dv, d = ev % dv;
+    st<T>(vbase + ((size_t)h * dv + d) * P + r, row[e] + (bias ? bias[e] : 0.f));
   }
 }
 
@@ -308,12 +310,13 @@ extern "C" int ti_qkv_prep_write(int dtype, const float* qkv, const float* bias,
   TI_REQUIRE(!inv_freq || (rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= dk),
              "qkv_prep_write: %d rotated entries do not fit a head of %d (even, at most the head)", rot_dims, dk);
   if (M == 0) return 0;
+  const dim3 grid(M, (n_head * dk + n_kv * (dk + dv) + 255) / 256);
   if (dtype == TI_F32)
-    qkv_prep_write_kernel<float><<<M, 256, 0, stream>>>(qkv, bias, inv_freq, rope_table, table_len, mag, rot_dims, pos, slot, table,
+    qkv_prep_write_kernel<float><<<grid, 256, 0, stream>>>(qkv, bias, inv_freq, rope_table, table_len, mag, rot_dims, pos, slot, table,
                                                         table_stride, (float*)pool, (float*)q_out, n_head, n_kv, dk, dv,
                                                         page_size, coef, every);
   else if (dtype == TI_BF16)
-    qkv_prep_write_kernel<bf16_t><<<M, 256, 0, stream>>>(qkv, bias, inv_freq, rope_table, table_len, mag, rot_dims, pos, slot, table,
+    qkv_prep_write_kernel<bf16_t><<<grid, 256, 0, stream>>>(qkv, bias, inv_freq, rope_table, table_len, mag, rot_dims, pos, slot, table,
                                                          table_stride, (bf16_t*)pool, (bf16_t*)q_out, n_head, n_kv, dk, dv,
                                                          page_size, coef, every);
   else
