@@ -233,7 +233,7 @@ __device__ __forceinline__ void finish_column(LatState<NRT>& st, const float* si
 
 // ------------------------------------------------------------------------------------------ tiles of a portion
 // tiles int32 [n][3] = (entry, first row, rows <= 64); entries int32 [.][4] = (row0, tokens, start, -).  qa [M][H][DK],
-// o [M][H][R].  Grid (tiles, heads), four wavefronts of 16 rows each.
+// o [M][H][R].  Grid (heads, tiles), four wavefronts of 16 rows each.
 template <int NKS, int NRT>
 __global__ void __launch_bounds__(256)
 latent_tiles_kernel(const bf16_t* __restrict__ qa, const bf16_t* __restrict__ pool, const int* __restrict__ table, int table_stride,
@@ -241,10 +241,10 @@ latent_tiles_kernel(const bf16_t* __restrict__ qa, const bf16_t* __restrict__ po
                     bf16_t* __restrict__ o, int H, int R, int DK, int P, size_t page_elems, float scale2, int window) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r16 = lane & 15;
-  const int e = tiles[3 * blockIdx.x], row0 = tiles[3 * blockIdx.x + 1] + 16 * wave;
-  const int n_rows = tiles[3 * blockIdx.x + 2] - 16 * wave;
+  const int e = tiles[3 * blockIdx.y], row0 = tiles[3 * blockIdx.y + 1] + 16 * wave;
+  const int n_rows = tiles[3 * blockIdx.y + 2] - 16 * wave;
   if (n_rows <= 0) return;
-  const int h = blockIdx.y;
+  const int h = blockIdx.x;
   const int e_row0 = entries[4 * e], e_n = entries[4 * e + 1], e_start = entries[4 * e + 2];
   const int kv_last = e_start + e_n - 1;
   const bool live = r16 < n_rows;
@@ -338,9 +338,9 @@ latent_tiles_lds_kernel(const bf16_t* __restrict__ qa, const bf16_t* __restrict_
   using S = LatStage<NKS, NRT>;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r16 = lane & 15;
-  const int e = tiles[3 * blockIdx.x], tile_row0 = tiles[3 * blockIdx.x + 1], tile_n = tiles[3 * blockIdx.x + 2];
+  const int e = tiles[3 * blockIdx.y], tile_row0 = tiles[3 * blockIdx.y + 1], tile_n = tiles[3 * blockIdx.y + 2];
   const int row0 = tile_row0 + 16 * wave, n_rows = tile_n - 16 * wave;      // a wavefront without rows still fetches and waits
-  const int h = blockIdx.y;
+  const int h = blockIdx.x;
   const int e_row0 = entries[4 * e], e_n = entries[4 * e + 1], e_start = entries[4 * e + 2];
   const int kv_last = e_start + e_n - 1;
   const bool live = r16 < n_rows;
@@ -482,7 +482,7 @@ latent_rows_merge_kernel(const float* __restrict__ part, const int* __restrict__
 // ------------------------------------------------------------------------------------------ the absorbed query
 // qa [M][H][DK] bf16: entries c < R: sum_k q[m, h, k] W_uk[h d + k, c], from w_uk_t [H][R][d] (a head's matrix transposed);
 // entries R + j: q_rot[m, h, j].  proj f32 [M, ld] holds the heads' queries [d + r] from column 0.  Grid (tokens / 16, heads,
-// R / 64): a wavefront takes one block of 16 latent entries.  A step of the sum beyond d reads the last one and counts as zero.
+// R / 256): a wavefront takes four blocks of 16 latent entries.  A step of the sum beyond d reads the last one and counts as zero.
 __global__ void __launch_bounds__(256)
 latent_absorb_mfma_kernel(const float* __restrict__ proj, int ldp, const bf16_t* __restrict__ w_uk_t, bf16_t* __restrict__ qa, int M,
                           int H, int d, int r, int R) {
@@ -492,23 +492,36 @@ latent_absorb_mfma_kernel(const float* __restrict__ proj, int ldp, const bf16_t*
   const int tok = blockIdx.x * 16 + r16;
   const bool live = tok < M;
   const float* q = proj + (size_t)(live ? tok : M - 1) * ldp + (size_t)h * (d + r);
-  const int ct = blockIdx.z * 4 + wave;
-  if (ct * 16 < R) {
-    const bf16_t* w = w_uk_t + ((size_t)h * R + ct * 16 + r16) * d;
-    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
+  // a wavefront takes four blocks of 16 latent entries: a step's query fragment is fetched once for the four
+  const int ct0 = (blockIdx.z * 4 + wave) * 4;
+  if (ct0 * 16 < R) {
+    const bf16_t* w[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) w[j] = w_uk_t + ((size_t)h * R + min((ct0 + j) * 16 + r16, R - 1)) * d;
+    floatx4 acc[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 2
     for (int k0 = 0; k0 < d; k0 += 32) {
       const int at = min(k0 + quad * 8, d - 8);
-      LFrag8 a, b;
-      a.u = *reinterpret_cast<const uint4*>(w + at);
+      const bool in = k0 + quad * 8 < d;
       const float4 x = *reinterpret_cast<const float4*>(q + at), y = *reinterpret_cast<const float4*>(q + at + 4);
+      LFrag8 b;
       b.u = make_uint4(pack_bf16x2(x.x, x.y), pack_bf16x2(x.z, x.w), pack_bf16x2(y.x, y.y), pack_bf16x2(y.z, y.w));
-      if (!(k0 + quad * 8 < d)) a.u = make_uint4(0u, 0u, 0u, 0u);
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc, 0, 0, 0);
+      if (!in) b.u = make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        LFrag8 a;
+        a.u = *reinterpret_cast<const uint4*>(w[j] + at);
+        acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc[j], 0, 0, 0);
+      }
     }
     if (live)
-      *reinterpret_cast<uint2*>(qa + ((size_t)tok * H + h) * DK + ct * 16 + quad * 4) =
-          make_uint2(pack_bf16x2(acc[0], acc[1]), pack_bf16x2(acc[2], acc[3]));
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if ((ct0 + j) * 16 < R)
+          *reinterpret_cast<uint2*>(qa + ((size_t)tok * H + h) * DK + (ct0 + j) * 16 + quad * 4) =
+              make_uint2(pack_bf16x2(acc[j][0], acc[j][1]), pack_bf16x2(acc[j][2], acc[j][3]));
   }
   if (blockIdx.z == 0) {
     const int n = min(16, M - (int)blockIdx.x * 16);
@@ -520,8 +533,8 @@ latent_absorb_mfma_kernel(const float* __restrict__ proj, int ldp, const bf16_t*
 }
 
 // ------------------------------------------------------------------------------------------ a head's weighted latent to its output
-// out [M][H dv] bf16: out[m, h dv + j] = sum_c o[m, h, c] W_uv[h dv + j, c].  Grid (tokens / 16, heads, dv / 64): a wavefront
-// takes one block of 16 outputs.
+// out [M][H dv] bf16: out[m, h dv + j] = sum_c o[m, h, c] W_uv[h dv + j, c].  Grid (tokens / 16, heads, dv / 128): a wavefront
+// takes two blocks of 16 outputs.
 __global__ void __launch_bounds__(256)
 latent_expand_mfma_kernel(const bf16_t* __restrict__ o, const bf16_t* __restrict__ w_uv, bf16_t* __restrict__ out, int M, int H, int R,
                           int dv) {
@@ -530,23 +543,33 @@ latent_expand_mfma_kernel(const bf16_t* __restrict__ o, const bf16_t* __restrict
   const int h = blockIdx.y;
   const int tok = blockIdx.x * 16 + r16;
   const bool live = tok < M;
-  const int jt = blockIdx.z * 4 + wave;
-  if (jt * 16 >= dv) return;
+  // a wavefront takes two blocks of 16 outputs: a step's fragment of the weighted latent is fetched once for both
+  const int jt0 = (blockIdx.z * 4 + wave) * 2;
+  if (jt0 * 16 >= dv) return;
   const bf16_t* orow = o + ((size_t)(live ? tok : M - 1) * H + h) * R;
-  const bf16_t* w = w_uv + ((size_t)h * dv + jt * 16 + r16) * R;
-  floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+  const bf16_t* w[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) w[j] = w_uv + ((size_t)h * dv + min((jt0 + j) * 16 + r16, dv - 1)) * R;
+  floatx4 acc[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll 4
   for (int c0 = 0; c0 < R; c0 += 32) {
     const int at = min(c0 + quad * 8, R - 8);
-    LFrag8 a, b;
-    a.u = *reinterpret_cast<const uint4*>(w + at);
+    LFrag8 b;
     b.u = *reinterpret_cast<const uint4*>(orow + at);
-    if (!(c0 + quad * 8 < R)) a.u = make_uint4(0u, 0u, 0u, 0u);
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc, 0, 0, 0);
+    if (!(c0 + quad * 8 < R)) b.u = make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      LFrag8 a;
+      a.u = *reinterpret_cast<const uint4*>(w[j] + at);
+      acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc[j], 0, 0, 0);
+    }
   }
   if (live)
-    *reinterpret_cast<uint2*>(out + (size_t)tok * H * dv + (size_t)h * dv + jt * 16 + quad * 4) =
-        make_uint2(pack_bf16x2(acc[0], acc[1]), pack_bf16x2(acc[2], acc[3]));
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      if ((jt0 + j) * 16 < dv)
+        *reinterpret_cast<uint2*>(out + (size_t)tok * H * dv + (size_t)h * dv + (jt0 + j) * 16 + quad * 4) =
+            make_uint2(pack_bf16x2(acc[j][0], acc[j][1]), pack_bf16x2(acc[j][2], acc[j][3]));
 }
 
 // ------------------------------------------------------------------------------------------ host
@@ -576,7 +599,7 @@ extern "C" int ti_latent_absorb_bf16(const float* proj, int ld, const void* w_uk
                  (d + r) % 4 == 0,
              "latent_absorb (bf16): bad sizes heads=%d dim=%d rot=%d rank=%d ld=%d", H, d, r, R, ld);
   if (M == 0) return 0;
-  latent_absorb_mfma_kernel<<<dim3((M + 15) / 16, H, (R + 63) / 64), 256, 0, stream>>>(proj, ld, (const bf16_t*)w_uk_t, (bf16_t*)qa, M, H, d, r, R);
+  latent_absorb_mfma_kernel<<<dim3((M + 15) / 16, H, (R + 255) / 256), 256, 0, stream>>>(proj, ld, (const bf16_t*)w_uk_t, (bf16_t*)qa, M, H, d, r, R);
   TI_LAUNCH_CHECK();
   return 0;
 }
@@ -584,7 +607,7 @@ extern "C" int ti_latent_absorb_bf16(const float* proj, int ld, const void* w_uk
 extern "C" int ti_latent_expand_bf16(const void* o, const void* w_uv, void* out, int M, int H, int R, int dv, hipStream_t stream) {
   TI_REQUIRE(H > 0 && H <= 65535 && R > 0 && R % 8 == 0 && dv > 0 && dv % 16 == 0, "latent_expand (bf16): bad sizes heads=%d rank=%d vdim=%d", H, R, dv);
   if (M == 0) return 0;
-  latent_expand_mfma_kernel<<<dim3((M + 15) / 16, H, (dv + 63) / 64), 256, 0, stream>>>((const bf16_t*)o, (const bf16_t*)w_uv, (bf16_t*)out, M, H, R, dv);
+  latent_expand_mfma_kernel<<<dim3((M + 15) / 16, H, (dv + 127) / 128), 256, 0, stream>>>((const bf16_t*)o, (const bf16_t*)w_uv, (bf16_t*)out, M, H, R, dv);
   TI_LAUNCH_CHECK();
   return 0;
 }
@@ -599,7 +622,10 @@ extern "C" int ti_latent_attention_tiles_bf16(const void* qa, const void* pool, 
              "latent_attention (tiles): heads=%d, a latent of %d + %d, pages of %d rows and %ld elements are not served", H, R, r,
              page_size, page_elems);
   if (n_tiles == 0) return 0;
-  const dim3 grid(n_tiles, H);
+  // heads along x: workgroups start in the order of the tiles' list, the ones that walk the most keys first, and the short
+  // ones fill the compute units as the long ones end
+  TI_REQUIRE(n_tiles <= 65535, "latent_attention (tiles): %d tiles in a step are not served", n_tiles);
+  const dim3 grid(H, n_tiles);
   // keys and latents shared through LDS (use_lds 0: every wavefront fetches its own, for tests and measurements); the two
   // stages of the largest sizes need more than the 64 KB a kernel may use without asking
 #define LA_TILES(K, V)                                                                                                              \
