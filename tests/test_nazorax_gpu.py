@@ -191,9 +191,9 @@ def latent_weights(rng, W, H, d, r, dv, R):
                                                    (8, 64, 32, 64, 128, 16, True), (16, 128, 64, 128, 512, 16, True)])
 def test_latent_attention_with_a_sink(ops, dtype, H, d, r, dv, R, P, scaling):
     """A whole request's projections prepared into the pages in two portions, then the attention of every row, against the
-    mixer of the plain implementation (its output projection the identity).  The latent of an early token is made large
-    before its norm (which takes that away again) and the key part of another one, which stays: a norm that is left out,
-    a far key that is lost and a sink that is forgotten all show."""
+    mixer of the plain implementation (its output projection the identity).  An early token's input is made large: its
+    latent loses that in its norm, its key part keeps it; a norm that is left out and a sink that is forgotten show.  (A far
+    key and a window's edge that stand out: the test of the matrix-core kernels below, whose row-wise run reads the same pages.)"""
     rng = np.random.default_rng(H * 100 + R)
     T, W, eps = (150 if R < 512 else 70), 48, 1e-5
     m = dict(heads=H, dim=d, rot_dim=r, vdim=dv, kv_rank=R, scale=1.2 / math.sqrt(d + r),
@@ -255,13 +255,25 @@ def test_latent_attention_on_the_matrix_cores(ops, H, d, r, dv, R, P, window):
              rot=dict(base=500.0, dims=r, scaling=nm.yarn(4.0, 32, 8.0, 1.0)))
     w = latent_weights(rng, W, H, d, r, dv, R)
     h = bf16_round(rng.normal(size=(T, W)))
-    h[2] *= 6.0
     nq = H * (d + r)
     proj = h @ np.concatenate([w["m.q"], w["m.dkv"]]).T
+    pos = np.arange(T, dtype=np.int32)
+    # One key is made to stand out for the last row of every head, through the projections themselves: the oldest key the
+    # window keeps (no window: the third token, far back among the others), and the key just behind the window gets the same
+    # latent, so that losing the first or seeing the second shows.
+    target = T - window if window else 2
+    if window:
+        proj[target - 1, nq:nq + R] = proj[target, nq:nq + R]
+    c_all = plain.rms_unit(proj[:, nq:nq + R], eps) * w["m.dkv.norm"]
+    for hd in range(H):                                     # the query: along the target's key, across what all keys share
+        k_all = c_all @ w["m.uk"][hd * d:(hd + 1) * d].T
+        dq = k_all[target] - k_all.mean(axis=0)
+        proj[T - 1, hd * (d + r):hd * (d + r) + d] = dq * (14.0 / (dq @ k_all[target] * m["scale"]))
+        proj[T - 1, hd * (d + r) + d:(hd + 1) * (d + r)] = 0.0
+    proj = proj.astype(np.float32).astype(np.float64)
     inv, tab, mag = rotation_inputs(m["rot"], 100)
     table, n_pages = paged(rng, T, P)
     pool = torch.full((n_pages, P, 2 * R + r), float("nan"), device="cuda", dtype=torch.bfloat16)      # rows never written hold anything
-    pos = np.arange(T, dtype=np.int32)
     slots = np.zeros(T, dtype=np.int32)
     pj = dev(proj)
     cut = 37
@@ -272,18 +284,18 @@ def test_latent_attention_on_the_matrix_cores(ops, H, d, r, dv, R, P, window):
     for t in (0, 1, P - 1, P, cut, T - 1):                  # the transposed latents are the rows' latents
         pg = flat[table[0, t // P]]
         assert np.array_equal(pg[:P * (R + r)].reshape(P, R + r)[t % P, :R], pg[P * (R + r):].reshape(R, P)[:, t % P]), t
-    if window:
-        want = np.zeros((T, H, dv))
-        q = proj[:, :nq].reshape(T, H, d + r)
-        c = bf16_round(plain.rms_unit(proj[:, nq:nq + R], eps) * w["m.dkv.norm"])
-        kr = bf16_round(plain.rotate_half(proj[:, nq + R:], pos, m["rot"]))
-        qr = plain.rotate_half(q[:, :, d:], pos, m["rot"])
-        vis = plain.window_mask(T, window)
-        for hd in range(H):
-            sc = (q[:, hd, :d] @ (c @ w["m.uk"][hd * d:(hd + 1) * d].T).T + qr[:, hd] @ kr.T) * m["scale"]
-            want[:, hd] = plain.softmax_rows(sc, vis, float(w["m.sink"][hd])) @ (c @ w["m.uv"][hd * dv:(hd + 1) * dv].T)
-    else:
-        want = plain.latent_attention(h, w, "m", m, eps).reshape(T, H, dv)
+    # the mixer's formulas on the projections, with what the pages hold rounded as the pages round it
+    want = np.zeros((T, H, dv))
+    q = proj[:, :nq].reshape(T, H, d + r)
+    c = bf16_round(plain.rms_unit(proj[:, nq:nq + R], eps) * w["m.dkv.norm"])
+    kr = bf16_round(plain.rotate_half(proj[:, nq + R:], pos, m["rot"]))
+    qr = plain.rotate_half(q[:, :, d:], pos, m["rot"])
+    vis = plain.window_mask(T, window or None)
+    for hd in range(H):
+        sc = (q[:, hd, :d] @ (c @ w["m.uk"][hd * d:(hd + 1) * d].T).T + qr[:, hd] @ kr.T) * m["scale"]
+        p_att = plain.softmax_rows(sc, vis, float(w["m.sink"][hd]))
+        assert (d < 16 or p_att[T - 1, target] > 0.2) and (not window or p_att[T - 1, target - 1] == 0.0)
+        want[:, hd] = p_att @ (c @ w["m.uv"][hd * dv:(hd + 1) * dv].T)
     uk, uv = dev(w["m.uk"], torch.bfloat16), dev(w["m.uv"], torch.bfloat16)
     uk_t = torch.empty(H * R, d, device="cuda", dtype=torch.bfloat16)
     ops.latent_transpose(uk, uk_t, H)
