@@ -61,6 +61,20 @@ def test_a_loop_from_the_first_layer_and_no_loop():
     assert "loop.in" not in Model(spec).tensors()
 
 
+def test_pages_of_a_latent_layer_hold_the_latents_twice_where_the_matrix_cores_serve_the_sizes():
+    """kv_rank + rot_dim numbers a token, and kv_rank more (the latents transposed) where the latent is a multiple of 16, latent and
+    key part together a multiple of 8, the unrotated query size a multiple of 8 and the value size a multiple of 16."""
+    from tinyinfer_amd.models.model import Model
+    _, spec = spec_of(nm.CONFIGS["wide"])
+    rows = [tuple(n.row_shape) for n, _ in Model(spec).cache_groups if type(n).__name__ == "PagedRowsNeed"]
+    assert rows == [(64 + 16 + 64,)]
+    config = copy.deepcopy(nm.CONFIGS["wide"])
+    config["layers"][1]["mixer"]["vdim"] = 40                # values that are no multiple of 16: rows only
+    _, spec = spec_of(config)
+    rows = [tuple(n.row_shape) for n, _ in Model(spec).cache_groups if type(n).__name__ == "PagedRowsNeed"]
+    assert rows == [(64 + 16,)]
+
+
 @pytest.mark.parametrize("change,word", [
     (lambda c: c.pop("width"), "width"),
     (lambda c: c["norm"].pop("eps"), "eps"),
