@@ -395,6 +395,7 @@ void ensure_builtin_architectures() {
     architectures().push_back({"Miterax", miterax_spec, miterax_typed_config});
     architectures().push_back({"Mumasun", mumasun_spec, mumasun_typed_config});
     architectures().push_back({"Nazorax", nazorax_spec, nazorax_typed_config});
+    architectures().push_back({"Dubozen", dubozen_spec, dubozen_typed_config});
   });
 }
 

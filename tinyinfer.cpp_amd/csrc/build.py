@@ -53,11 +53,12 @@ ON_DEMAND = ("measure",)
 
 # libraries that only some architectures call into (by the name config.json gives the architecture); every other
 # library serves them all
-ONLY_FOR = {"pointwise": ("Miterax", "Nazorax"), "recurrent": ("Miterax",), "residual": ("Mumasun",), "diff_attention": ("Mumasun",),
-            "diff_attention_bf16": ("Mumasun",), "moe": ("Mumasun", "Nazorax"), "moe_bf16": ("Mumasun", "Nazorax"),
-            "latent_attention": ("Nazorax",), "latent_attention_bf16": ("Nazorax",)}
+ONLY_FOR = {"pointwise": ("Miterax", "Nazorax", "Dubozen"), "recurrent": ("Miterax",), "residual": ("Mumasun",), "diff_attention": ("Mumasun",),
+            "diff_attention_bf16": ("Mumasun",), "moe": ("Mumasun", "Nazorax", "Dubozen"), "moe_bf16": ("Mumasun", "Nazorax", "Dubozen"),
+            "latent_attention": ("Nazorax",), "latent_attention_bf16": ("Nazorax",), "hyper": ("Dubozen",),
+            "gated_attention": ("Dubozen",), "linear_attention": ("Dubozen",)}
 # ... and libraries that a named architecture never calls into
-NOT_FOR = {"attention_generic": ("Mumasun",), "attention_bf16": ("Mumasun",)}
+NOT_FOR = {"attention_generic": ("Mumasun", "Dubozen"), "attention_bf16": ("Mumasun", "Dubozen")}
 
 
 def libraries_for(dtype: str, architecture: str = None) -> List[str]:
@@ -91,7 +92,7 @@ def architecture_of(model_dir: str):
 # the host library (configuration, weights, parts, cache manager, step function, scheduler, sampler
 # and the C interface the Python package binds): C++17, no device code
 PKG = os.path.dirname(HERE)
-HOST_SOURCES = ["config/json.cpp", "config/config.cpp", "config/miterax.cpp", "config/mumasun.cpp", "config/nazorax.cpp", "ops/ops.cpp", "parts/parts.cpp", "weights/weights.cpp",
+HOST_SOURCES = ["config/json.cpp", "config/config.cpp", "config/miterax.cpp", "config/mumasun.cpp", "config/nazorax.cpp", "config/dubozen.cpp", "ops/ops.cpp", "parts/parts.cpp", "weights/weights.cpp",
                 "models/model.cpp", "cache/cache_manager.cpp", "engine/engine.cpp", "engine/scheduler.cpp",
                 "sampling/sampler.cpp", "engine/c_api.cpp"]
 HOST_HEADERS = ["include/inference.h", "weights/weights.h", "csrc/tinyinfer_kernels.h"]

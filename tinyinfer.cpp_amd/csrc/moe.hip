@@ -63,9 +63,13 @@ __device__ __forceinline__ float wave_dot(FA fa, const T* __restrict__ b, int n,
 template <typename T, bool VEC>
 __global__ void __launch_bounds__(256)
 moe_route_kernel(const T* __restrict__ h, const float* __restrict__ router, int* __restrict__ ids, float* __restrict__ wts,
-                 int W, int E, int top, int score_kind, int renormalize) {
+                 int W, int E, int top, int score_kind, int renormalize, const float* __restrict__ correction = nullptr,
+                 int n_groups = 0, int keep = 0, float weight_scale = 1.f, float sum_floor = 0.f) {
   __shared__ float s_score[MOE_MAX_EXPERTS];
+  __shared__ float s_plain[MOE_MAX_EXPERTS];      // the scores the weights are taken from, where the choice reads corrected ones
+  __shared__ float s_group[MOE_MAX_EXPERTS];
   __shared__ float red[4];
+  const bool corrected = correction != nullptr || n_groups > 1;
   const int m = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const T* row = h + (size_t)m * W;
@@ -86,6 +90,40 @@ moe_route_kernel(const T* __restrict__ h, const float* __restrict__ router, int*
     for (int e = threadIdx.x; e < E; e += 256) s_score[e] = 1.0f / (1.0f + expf(-s_score[e]));
   }
   __syncthreads();
+  if (corrected) {
+    // the choice reads score + correction; the weights keep the score itself
+    for (int e = threadIdx.x; e < E; e += 256) {
+      s_plain[e] = s_score[e];
+      if (correction) s_score[e] += correction[e];
+    }
+    __syncthreads();
+    if (n_groups > 1) {
+      // groups of E / n_groups neighbours: a group's score is the sum of its two largest choice scores; experts outside
+      // the `keep` best groups (ties to the lower group) cannot be chosen
+      const int per = E / n_groups;
+      for (int g = threadIdx.x; g < n_groups; g += 256) {
+        float a = -INFINITY, b = -INFINITY;
+        for (int e = g * per; e < (g + 1) * per; ++e) {
+          const float s = s_score[e];
+          if (s > a) {
+            b = a;
+            a = s;
+          } else if (s > b) {
+            b = s;
+          }
+        }
+        s_group[g] = per > 1 ? a + b : a;
+      }
+      __syncthreads();
+      for (int g = threadIdx.x; g < n_groups; g += 256) {
+        int better = 0;
+        for (int o = 0; o < n_groups; ++o) better += (s_group[o] > s_group[g] || (s_group[o] == s_group[g] && o < g)) ? 1 : 0;
+        if (better >= keep)
+          for (int e = g * per; e < (g + 1) * per; ++e) s_score[e] = -INFINITY;
+      }
+      __syncthreads();
+    }
+  }
   if (wave != 0) return;
   float total = 0.f, first = 0.f;
   for (int k = 0; k < top; ++k) {
@@ -107,6 +145,7 @@ moe_route_kernel(const T* __restrict__ h, const float* __restrict__ router, int*
         at = oa;
       }
     }
+    if (corrected) best = s_plain[at];
     if (lane == 0) {
       ids[(size_t)m * top + k] = at;
       wts[(size_t)m * top + k] = best;
@@ -124,11 +163,24 @@ moe_route_kernel(const T* __restrict__ h, const float* __restrict__ router, int*
     __builtin_amdgcn_wave_barrier();
     __threadfence_block();
   }
-  if ((renormalize || score_kind == MOE_SOFTMAX_CHOSEN) && lane < top) wts[(size_t)m * top + lane] /= total;
+  if ((renormalize || score_kind == MOE_SOFTMAX_CHOSEN) && lane < top) wts[(size_t)m * top + lane] /= total + sum_floor;
+  if (weight_scale != 1.f && lane < top) wts[(size_t)m * top + lane] *= weight_scale;
 }
 
 extern "C" int ti_moe_route(int dtype, const void* h, const float* router, int* ids, float* wts, int M, int W, int E, int top,
                             int score_kind, int renormalize, hipStream_t stream) {
+  return ti_moe_route_grouped(dtype, h, router, nullptr, ids, wts, M, W, E, top, score_kind, renormalize, 0, 0, 1.f, 0.f, stream);
+}
+
+// the same with what a grouped router adds: `correction` f32 [E] (null: none) joins the scores for the choice only; the experts
+// form n_groups groups of neighbours of which the `keep` best may be chosen from (n_groups <= 1: no groups); the weights are
+// the chosen experts' uncorrected scores, divided by their sum + sum_floor where `renormalize`, times weight_scale
+extern "C" int ti_moe_route_grouped(int dtype, const void* h, const float* router, const float* correction, int* ids, float* wts,
+                                    int M, int W, int E, int top, int score_kind, int renormalize, int n_groups, int keep,
+                                    float weight_scale, float sum_floor, hipStream_t stream) {
+  TI_REQUIRE(n_groups <= 1 || (E % n_groups == 0 && keep >= 1 && keep <= n_groups && (long)keep * (E / n_groups) >= top),
+             "moe_route: %d groups of which %d are kept do not fit %d experts and top %d", n_groups, keep, E, top);
+  TI_REQUIRE((!correction && n_groups <= 1) || score_kind != MOE_SOFTMAX_CHOSEN, "moe_route: a correction or groups do not go with weights from the chosen logits");
   TI_REQUIRE(M >= 0 && W > 0 && E > 0 && E <= MOE_MAX_EXPERTS && top > 0 && top <= E && top <= MOE_MAX_TOP,
              "moe_route: bad sizes M=%d W=%d experts=%d top=%d (up to %d experts, top up to %d)", M, W, E, top, MOE_MAX_EXPERTS,
              MOE_MAX_TOP);
@@ -136,7 +188,7 @@ extern "C" int ti_moe_route(int dtype, const void* h, const float* router, int* 
   if (M == 0) return 0;
   const int piece = dtype == TI_F32 ? 4 : 8;
   const bool vec = W % piece == 0 && ((uintptr_t)h & 15) == 0;
-#define MOE_ROUTE(T, V) moe_route_kernel<T, V><<<M, 256, 0, stream>>>((const T*)h, router, ids, wts, W, E, top, score_kind, renormalize)
+#define MOE_ROUTE(T, V) moe_route_kernel<T, V><<<M, 256, 0, stream>>>((const T*)h, router, ids, wts, W, E, top, score_kind, renormalize, correction, n_groups, keep, weight_scale, sum_floor)
   if (dtype == TI_F32) {
     if (vec) MOE_ROUTE(float, true);
     else MOE_ROUTE(float, false);

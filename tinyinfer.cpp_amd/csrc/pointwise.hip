@@ -352,6 +352,7 @@ extern "C" int ti_dyt(int out_dtype, const float* x, const float* alpha, const f
 // z f32 [R, 2F] = [gate | up] (rows ldz floats apart), bias f32 [2F] (null: none) added first.
 //   kind 0: out = silu(g) * u
 //   kind 1: g = min(g, limit), u = clamp(u, -limit, limit); out = g * sigmoid(alpha g) * (u + 1)
+//   kind 2: out = gelu(g) * u, gelu in its tanh form: g / 2 (1 + tanh(sqrt(2 / pi) (g + 0.044715 g^3)))
 __device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
 
 template <typename T>
@@ -369,6 +370,8 @@ __global__ void gated_act_kernel(const float* __restrict__ z, long ldz, const fl
     float y;
     if (kind == 0) {
       y = g * sigmoid_f(g) * u;
+    } else if (kind == 2) {
+      y = 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))) * u;
     } else {
       g = fminf(g, limit);
       u = fminf(fmaxf(u, -limit), limit);
@@ -380,7 +383,7 @@ __global__ void gated_act_kernel(const float* __restrict__ z, long ldz, const fl
 
 extern "C" int ti_gated_act(int out_dtype, const float* z, long ldz, const float* bias, void* out, long R, int F, int kind,
                             float limit, float alpha, hipStream_t stream) {
-  TI_REQUIRE(R >= 0 && F > 0 && ldz >= 2L * F && (kind == 0 || kind == 1), "gated_act: bad sizes R=%ld F=%d ld=%ld kind=%d", R, F, ldz, kind);
+  TI_REQUIRE(R >= 0 && F > 0 && ldz >= 2L * F && (kind >= 0 && kind <= 2), "gated_act: bad sizes R=%ld F=%d ld=%ld kind=%d", R, F, ldz, kind);
   if (R == 0) return 0;
   const long n = R * F;
   const unsigned blocks = (unsigned)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);

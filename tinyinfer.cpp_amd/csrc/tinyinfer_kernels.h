@@ -191,6 +191,44 @@ int ti_mlstm_scan_chunked(const float* proj, int ld, int off_q, int off_k, int o
 int ti_gated_head_norm(int out_dtype, const float* o, const float* gate, int ld, int off_g, const float* w, void* out,
                        int M, int heads, int dv, float eps, hipStream_t stream);
 
+// ---- libti_hyper: the layer norm, and a residual kept in several streams
+// out[r] = layernorm(sum_s coef[s] x_s[rows ? rows[r] : r]) * w (mean and variance, no bias), in `out_dtype`; the streams lie
+// stream_stride floats apart; coef null: the first stream alone.  out may be x (float32, one stream).  H up to 16384
+int ti_mixed_layernorm(int out_dtype, const float* x, long stream_stride, int S, const float* coef, const int* rows,
+                       const float* w, void* out, int n_rows, int H, float eps, hipStream_t stream);
+// u[i] = sum_s coef[s] x_s[i] (coef null: the plain sum)
+int ti_hyper_combine(const float* x, long stream_stride, int S, const float* coef, float* u, long n, hipStream_t stream);
+// every stream a copy of x
+int ti_hyper_spread(const float* x, float* streams, long stream_stride, int S, long n, hipStream_t stream);
+// x_t <- sum_s mix[s, t] x_s + back[t] y, every t at once from the old streams
+int ti_hyper_write(float* streams, long stream_stride, int S, const float* mix, const float* back, const float* y, long n,
+                   hipStream_t stream);
+
+// ---- libti_gated_attention: attention with per-head norms, values from the keys or mixed with another layer's, a sink, a gate
+// proj f32 [M, ld] holds q (n_head x dk), k (n_kv x dk) and v (n_kv x dv; off_v < 0: the values are the keys as projected) from
+// the given columns on.  q_w / k_w (null: none): RMS norm of every head before the rotation of its first rot_dims entries.
+// mix_mode 1: the values also go to v_kept f32 [M, n_kv dv]; 2: v <- (1 - lambda) v + lambda v_kept (lambda: one float in
+// device memory).  q to q_out, k and v into the pages K [n_kv][P][dk] | V [n_kv][dv][P]
+int ti_gated_qkv_prep(int dtype, const float* proj, int ld, int off_q, int off_k, int off_v, const float* q_w, const float* k_w,
+                      float eps, const float* inv_freq, const float* rope_table, int table_len, float mag, int rot_dims,
+                      int mix_mode, const float* mix_lambda, float* v_kept, const int* pos, const int* slot, const int* table,
+                      int table_stride, void* pool, void* q_out, int M, int n_head, int n_kv, int dk, int dv, int page_size,
+                      hipStream_t stream);
+// causal softmax attention of every row over such pages; sink f32 [n_head] (null: none) joins the denominator; gate (null:
+// none) f32 rows of gate_ld floats, the output times sigmoid of entry h dv + d (gate_mode 1) or h (gate_mode 2)
+int ti_gated_attention_rows(int dtype, const void* q, const void* pool, const int* table, int table_stride, const int* pos,
+                            const int* slot, const float* sink, const float* gate, int gate_ld, int gate_mode, void* out, int M,
+                            int n_head, int n_kv, int dk, int dv, int page_size, float scale, int window, hipStream_t stream);
+
+// ---- libti_linear_attention: linear attention with a fixed decay per head, and the gated norm behind it
+// S_t = decay_h S_(t-1) + k_t v_t^T, o_t = S_t^T q_t with q, k, v = silu of the given columns of proj f32 [M, ld]; state f32
+// [slots][heads][dk][dv]; entry_meta [n_entries][4] = (row0, tokens, start, slot); o f32 [M, heads dv]
+int ti_decay_scan(const float* proj, int ld, int off_q, int off_k, int off_v, const float* decay, float* state, long slot_stride,
+                  const int* entry_meta, int n_entries, float* o, int heads, int dk, int dv, hipStream_t stream);
+// out = o / rms(o over the whole row) * w * sigmoid(gate), gate in rows of ld floats from column off_g on
+int ti_gated_row_norm(int out_dtype, const float* o, const float* gate, int ld, int off_g, const float* w, void* out, int M, int W,
+                      float eps, hipStream_t stream);
+
 // ---- libti_residual: layers that norm what a sublayer returns
 // x[m] (+)= y'[m] / sqrt(mean(y'[m]^2) + eps) * g; y'[m] = y[m], or with `gather` (int32 [M][n_gather]) the sum of
 // the rows y[gather[m][k]] in ascending k (gather null and n_gather > 1: of the rows y[m n_gather + k]).  accumulate 0: x is overwritten (y may be x itself).  rounded (may be null):
@@ -248,6 +286,13 @@ long ti_diff_attention_rows_scratch(int n_rows, int n_kv, int dv, int n_splits);
 // largest per token (ties: the lower index) to ids int32 [M, top] and wts f32 [M, top] (renormalize: divided by their sum)
 int ti_moe_route(int dtype, const void* h, const float* router, int* ids, float* wts, int M, int W, int E, int top,
                  int score_kind, int renormalize, hipStream_t stream);
+// the same for a grouped router: correction f32 [E] (null: none) joins the scores for the choice only; the experts form
+// n_groups groups of neighbours, a group's score the sum of its two largest choice scores, and only experts of the `keep`
+// best groups can be chosen (n_groups <= 1: no groups); weights: the chosen experts' uncorrected scores, divided by their
+// sum + sum_floor where `renormalize`, times weight_scale
+int ti_moe_route_grouped(int dtype, const void* h, const float* router, const float* correction, int* ids, float* wts, int M,
+                         int W, int E, int top, int score_kind, int renormalize, int n_groups, int keep, float weight_scale,
+                         float sum_floor, hipStream_t stream);
 // y f32 [M, W] = sum_k down[e_k] relu(up[e_k] (s_k h))^2 (scale_input) or sum_k s_k down[e_k] relu(up[e_k] h)^2;
 // up [E][F][W], down [E][W][F] in the dtype of h; act: scratch of that dtype, [M top][F]; part: f32 [M top][W].  A workgroup
 // per expert and 16 outputs walks its weights once for all the pairs that chose the expert: steps of few tokens, and float32.

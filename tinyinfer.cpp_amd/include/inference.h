@@ -169,6 +169,9 @@ ModelSpec mumasun_spec(const Json& config);
 // the Nazorax decoder (config/nazorax.cpp)
 Json nazorax_typed_config(const Json& config);
 ModelSpec nazorax_spec(const Json& config);
+// the Dubozen decoder (config/dubozen.cpp)
+Json dubozen_typed_config(const Json& config);
+ModelSpec dubozen_spec(const Json& config);
 // {"architecture": the registered name that matched, "config": the typed configuration (the input itself if
 // the architecture registered no reader)}; ConfigError as spec_from_config
 Json typed_config(const Json& config);
@@ -361,7 +364,8 @@ class Ops {
   void dyt(const Tensor& x, const Tensor& alpha, const Tensor& w, const Tensor& b, const Tensor& out, const int* rows = nullptr,
            int64_t n_rows = 0);
   // z f32 [R, 2F] = [gate | up] (+ bias f32 [2F], may be undefined) -> out [R, F] in its own dtype
-  enum GatedAct { Silu = 0, ClampedGlu = 1 };   // silu(g) u;  g = min(g, limit), u = clamp(u, -limit, limit): g sigmoid(alpha g) (u + 1)
+  // silu(g) u;  g = min(g, limit), u = clamp(u, -limit, limit): g sigmoid(alpha g) (u + 1);  gelu(g) u with gelu's tanh form
+  enum GatedAct { Silu = 0, ClampedGlu = 1, GeluTanh = 2 };
   void gated_act(const Tensor& z, const Tensor& bias, const Tensor& out, GatedAct kind, float limit = 0.f, float alpha = 1.f);
   // out [M, 2H] = [a | b] in out's dtype
   void concat_round(const Tensor& a, const Tensor& b, const Tensor& out);
@@ -388,6 +392,38 @@ class Ops {
   void latent_transpose(const Tensor& src, const Tensor& dst, int heads);
   // whether the matrix-core kernels serve these sizes
   bool latent_fast(int heads, int dim, int rot_dim, int rank, int v_dim, int page_size);
+  // ---- the layer norm; a residual kept in several streams; gated attention; linear attention with a fixed decay
+  // out[r] = layernorm(x[rows ? rows[r] : r]) * w: mean and variance (of the deviations), a gain, no bias; out may be x (float32)
+  void layernorm(const Tensor& x, const Tensor& w, float eps, const Tensor& out, const int* rows = nullptr, int64_t n_rows = 0);
+  // the same of u = sum_s coef[s] streams[s] (streams f32 [S, M, H], coef f32 [S]) without forming u
+  void layernorm_mixed(const Tensor& streams, const Tensor& coef, const Tensor& w, float eps, const Tensor& out);
+  // u f32 [M, H] = sum_s coef[s] streams[s] (coef undefined: the plain sum)
+  void hyper_combine(const Tensor& streams, const Tensor& coef, const Tensor& u);
+  void hyper_spread(const Tensor& x, const Tensor& streams);                       // every stream a copy of x
+  // streams[t] <- sum_s mix[s, t] streams[s] + back[t] y, every t at once from the old streams (mix f32 [S, S], back f32 [S])
+  void hyper_write(const Tensor& streams, const Tensor& mix, const Tensor& back, const Tensor& y);
+  // What a gated attention layer does to the 32-bit sums of its stacked projection before the attention itself: proj f32 [M, N]
+  // holds q (heads x dk), k (kv_heads x dk) and v (kv_heads x dv) from the given columns on (off_v < 0: the values are the keys as
+  // projected, before norm and rotation).  q_w / k_w (undefined: none): an RMS norm of every head with a weight of dk shared by the
+  // heads, before the rotation.  mix_mode 1: this layer's values are also kept in v_kept f32 [M, kv_heads dv] for later layers; 2:
+  // v <- (1 - lambda) v + lambda v_kept, lambda f32 [1].  q to q_out, k and v into the pages (K [kv][P][dk] | V [kv][dv][P])
+  struct QkvColumns { int q = 0, k = 0, v = -1; };
+  struct ValueMix { int mode = 0; Tensor lambda, kept; };
+  void gated_qkv_prep(const Tensor& proj, const QkvColumns& cols, const Tensor& q_w, const Tensor& k_w, float eps, const Rotation& rot,
+                      const ValueMix& mix, const int* positions, const int* slots, const CacheView& view, const Tensor& pool,
+                      const Tensor& q_out, int heads, int kv_heads, int dk, int dv);
+  // causal softmax attention over such pages with a sink (f32 [heads], undefined: none) in the denominator and a sigmoid gate on
+  // the output read from proj's columns from gate_col on: gate_mode 1 one number an output entry, 2 one a head (0: no gate)
+  struct AttentionGate { Tensor proj; int col = 0, mode = 0; };
+  void gated_attention(const Tensor& q, const Tensor& pool, const CacheView& view, const int* positions, const int* slots,
+                       const Tensor& sink, const AttentionGate& gate, const Tensor& out, int heads, int kv_heads, int dk, int dv,
+                       float scale, int window);
+  // Linear attention with a fixed decay per head over each entry's tokens, from and into its state slot: S <- decay_h S + k v^T,
+  // o = S^T q with q, k, v = silu of proj's columns; decay f32 [heads]; state f32 [slots][heads][dk dv]; o f32 [M, heads dv]
+  void decay_scan(const Tensor& proj, const QkvColumns& cols, const Tensor& decay, const Tensor& state, const int* entry_meta,
+                  int n_entries, const Tensor& o, int heads, int dk, int dv);
+  // out = o / rms(o over the whole row) * w * sigmoid(gate columns of proj), in the compute dtype
+  void gated_row_norm(const Tensor& o, const Tensor& proj, int gate_col, const Tensor& w, float eps, const Tensor& out);
   // ---- layers that norm what a sublayer returns; short convolutions; differential attention; mixtures of experts
   // x (+)= y / rms(y) * gain (32-bit; gain is the factor itself).  accumulate false: x is overwritten (y may be x).
   // gather (device int32 [M][n_gather]): row m of y is the sum of the rows y[gather[m][k]], k ascending; no list and
@@ -424,6 +460,13 @@ class Ops {
   // the `top` experts with the largest scores of h against router f32 [E, W]: ids int32 [M, top], wts f32 [M, top]
   void moe_route(const Tensor& h, const Tensor& router, const Tensor& ids, const Tensor& wts, int top, RouterScore score,
                  bool renormalize);
+  // a grouped router: `correction` f32 [E] (undefined: none) joins the scores for the choice only; the experts form `groups`
+  // groups of neighbours (a group's score: the sum of its two largest choice scores) and only experts of the `keep` best groups
+  // can be chosen (groups <= 1: none); the weights are the chosen experts' uncorrected scores, divided by their sum + sum_floor
+  // where `renormalize`, times weight_scale
+  struct RouterGroups { Tensor correction; int groups = 0, keep = 0; float weight_scale = 1.f, sum_floor = 0.f; };
+  void moe_route(const Tensor& h, const Tensor& router, const Tensor& ids, const Tensor& wts, int top, RouterScore score,
+                 bool renormalize, const RouterGroups& grouped);
   // y f32 [M, W] = sum over a token's experts of down_e relu(up_e h)^2, the weight on the expert's input or output;
   // up [E F, W], down [E W, F]; scratch comes from `ws`.  With `rows` (and bfloat16, many tokens, sizes the matrix-core kernels
   // take) y may stay unwritten: then rows->t is f32 [M top, W] and rows->gather device int32 [M][top]: row m of the result is
@@ -660,7 +703,11 @@ class NormPart : public Part { public: using Part::Part; const char* family() co
   virtual bool can_add() const { return false; }
   // rounded (may be null): also receives the new x in its own dtype
   virtual void forward_add(StepContext& ctx, const Tensor& y, const Tensor& x, bool accumulate, const int* gather = nullptr,
-                           int n_gather = 0, const Tensor* rounded = nullptr); };
+                           int n_gather = 0, const Tensor* rounded = nullptr);
+  // the norm of u = sum_s coef[s] streams[s] (streams f32 [S, M, dim], coef f32 [S]) without u being formed: for arrangements
+  // that keep the residual in several streams
+  virtual bool can_mix() const { return false; }
+  virtual Rows forward_mixed(StepContext& ctx, const Tensor& streams, const Tensor& coef); };
 class PositionPart : public Part { public: using Part::Part; const char* family() const override { return "pos"; }
   virtual bool fused(Ops::Rotation& rot) const { return false; }    // arguments for the fused q/k kernels
   virtual bool additive() const { return false; }                   // an encoding added to the residual behind the embedding ...

@@ -1167,6 +1167,150 @@ void Ops::gated_head_norm(const Tensor& o, const Tensor& proj, int gate_col, con
   check("recurrent", rc, "gated_head_norm");
 }
 
+// ------------------------------------------------- the layer norm, streams of a residual, gated attention, decayed linear attention
+void Ops::layernorm(const Tensor& x, const Tensor& w, float eps, const Tensor& out, const int* rows, int64_t n_rows) {
+  TIMED("layernorm " + std::to_string(rows ? n_rows : x.shape[0]) + "x" + std::to_string(x.shape[1]));
+  require(x.ndim == 2 && x.dtype == DType::F32 && x.contiguous(), "layernorm: x must be a contiguous float32 matrix");
+  const int64_t H = x.shape[1], n = rows ? n_rows : x.shape[0];
+  require(w.dtype == DType::F32 && w.numel() == H, "layernorm: w " + w.describe() + " does not fit width " + std::to_string(H));
+  require(out.ndim == 2 && out.shape[0] == n && out.shape[1] == H && out.contiguous(), "layernorm: out " + out.describe() + " does not fit");
+  int rc = KERNEL("hyper", ti_mixed_layernorm)(code(out.dtype, "layernorm"), (const float*)x.data, 0L, 1, nullptr, rows, (const float*)w.data,
+                                               out.data, (int)n, (int)H, eps, (hipStream_t)launch_stream());
+  check("hyper", rc, "layernorm");
+}
+
+static void check_streams(const char* what, const Tensor& streams) {
+  require(streams.ndim == 3 && streams.dtype == DType::F32 && streams.contiguous() && streams.shape[0] >= 1,
+          std::string(what) + ": streams " + streams.describe() + " must be contiguous float32 [S, M, H]");
+}
+
+void Ops::layernorm_mixed(const Tensor& streams, const Tensor& coef, const Tensor& w, float eps, const Tensor& out) {
+  TIMED("layernorm_mixed " + dims(streams));
+  check_streams("layernorm_mixed", streams);
+  const int64_t S = streams.shape[0], M = streams.shape[1], H = streams.shape[2];
+  require(coef.dtype == DType::F32 && coef.numel() == S && w.dtype == DType::F32 && w.numel() == H,
+          "layernorm_mixed: coef " + coef.describe() + " or w " + w.describe() + " do not fit");
+  require(out.ndim == 2 && out.shape[0] == M && out.shape[1] == H && out.contiguous(), "layernorm_mixed: out " + out.describe() + " does not fit");
+  int rc = KERNEL("hyper", ti_mixed_layernorm)(code(out.dtype, "layernorm_mixed"), (const float*)streams.data, (long)(M * H), (int)S,
+                                               (const float*)coef.data, nullptr, (const float*)w.data, out.data, (int)M, (int)H, eps,
+                                               (hipStream_t)launch_stream());
+  check("hyper", rc, "layernorm_mixed");
+}
+
+void Ops::hyper_combine(const Tensor& streams, const Tensor& coef, const Tensor& u) {
+  TIMED("hyper_combine " + dims(streams));
+  check_streams("hyper_combine", streams);
+  const int64_t S = streams.shape[0], n = streams.shape[1] * streams.shape[2];
+  require((!coef.defined() || (coef.dtype == DType::F32 && coef.numel() == S)) && u.dtype == DType::F32 && u.contiguous() && u.numel() == n,
+          "hyper_combine: coef " + coef.describe() + " or u " + u.describe() + " do not fit");
+  int rc = KERNEL("hyper", ti_hyper_combine)((const float*)streams.data, (long)n, (int)S, coef.defined() ? (const float*)coef.data : nullptr,
+                                             (float*)u.data, (long)n, (hipStream_t)launch_stream());
+  check("hyper", rc, "hyper_combine");
+}
+
+void Ops::hyper_spread(const Tensor& x, const Tensor& streams) {
+  TIMED("hyper_spread " + dims(streams));
+  check_streams("hyper_spread", streams);
+  const int64_t n = streams.shape[1] * streams.shape[2];
+  require(x.dtype == DType::F32 && x.contiguous() && x.numel() == n, "hyper_spread: x " + x.describe() + " does not fit");
+  int rc = KERNEL("hyper", ti_hyper_spread)((const float*)x.data, (float*)streams.data, (long)n, (int)streams.shape[0], (long)n,
+                                            (hipStream_t)launch_stream());
+  check("hyper", rc, "hyper_spread");
+}
+
+void Ops::hyper_write(const Tensor& streams, const Tensor& mix, const Tensor& back, const Tensor& y) {
+  TIMED("hyper_write " + dims(streams));
+  check_streams("hyper_write", streams);
+  const int64_t S = streams.shape[0], n = streams.shape[1] * streams.shape[2];
+  require(mix.dtype == DType::F32 && mix.numel() == S * S && mix.contiguous() && back.dtype == DType::F32 && back.numel() == S &&
+              y.dtype == DType::F32 && y.contiguous() && y.numel() == n,
+          "hyper_write: mix " + mix.describe() + ", back " + back.describe() + " or y " + y.describe() + " do not fit");
+  int rc = KERNEL("hyper", ti_hyper_write)((float*)streams.data, (long)n, (int)S, (const float*)mix.data, (const float*)back.data,
+                                           (const float*)y.data, (long)n, (hipStream_t)launch_stream());
+  check("hyper", rc, "hyper_write");
+}
+
+void Ops::gated_qkv_prep(const Tensor& proj, const QkvColumns& cols, const Tensor& q_w, const Tensor& k_w, float eps, const Rotation& rot,
+                         const ValueMix& mix, const int* positions, const int* slots, const CacheView& view, const Tensor& pool,
+                         const Tensor& q_out, int heads, int kv_heads, int dk, int dv) {
+  TIMED("gated_qkv_prep " + dims(proj) + (q_w.defined() ? " norm" : "") + (rot.inv_freq ? " rotation" : "") +
+        (cols.v < 0 ? " v=k" : "") + (mix.mode ? " mix" + std::to_string(mix.mode) : ""));
+  require(proj.ndim == 2 && proj.dtype == DType::F32 && proj.contiguous(), "gated_qkv_prep: proj must be contiguous float32 [M, N]");
+  const int64_t M = proj.shape[0];
+  require(q_out.ndim == 2 && q_out.shape[0] == M && q_out.shape[1] == (int64_t)heads * dk && q_out.contiguous(),
+          "gated_qkv_prep: q_out has the wrong shape");
+  require((!q_w.defined() || (q_w.dtype == DType::F32 && q_w.numel() == dk)) && (!k_w.defined() || (k_w.dtype == DType::F32 && k_w.numel() == dk)),
+          "gated_qkv_prep: the heads' norm weights must be float32 [" + std::to_string(dk) + "]");
+  require(mix.mode == 0 || (mix.kept.dtype == DType::F32 && mix.kept.contiguous() && mix.kept.numel() == M * kv_heads * dv &&
+                            (mix.mode == 1 || (mix.lambda.dtype == DType::F32 && mix.lambda.numel() == 1))),
+          "gated_qkv_prep: the kept values " + mix.kept.describe() + " or the factor do not fit");
+  check_split_pool("gated_qkv_prep", pool, kv_heads, dk, dv, q_out.dtype);
+  const int rot_dims = rot.inv_freq ? (rot.dims > 0 ? rot.dims : dk) : 0;
+  int rc = KERNEL("gated_attention", ti_gated_qkv_prep)(
+      code(q_out.dtype, "gated_qkv_prep"), (const float*)proj.data, (int)proj.shape[1], cols.q, cols.k, cols.v,
+      q_w.defined() ? (const float*)q_w.data : nullptr, k_w.defined() ? (const float*)k_w.data : nullptr, eps, rot.inv_freq, rot.table,
+      rot.table_len, rot.mag, rot_dims, mix.mode, mix.mode == 2 ? (const float*)mix.lambda.data : nullptr,
+      mix.mode ? (float*)mix.kept.data : nullptr, positions, slots, view.table, view.table_width, pool.data, q_out.data, (int)M, heads,
+      kv_heads, dk, dv, (int)pool.shape[2], (hipStream_t)launch_stream());
+  check("gated_attention", rc, "gated_qkv_prep");
+}
+
+void Ops::gated_attention(const Tensor& q, const Tensor& pool, const CacheView& view, const int* positions, const int* slots,
+                          const Tensor& sink, const AttentionGate& gate, const Tensor& out, int heads, int kv_heads, int dk, int dv,
+                          float scale, int window) {
+  TIMED("gated_attention " + dims(q) + (sink.defined() ? " sink" : "") + (gate.mode ? " gate" + std::to_string(gate.mode) : ""));
+  const int64_t M = q.shape[0];
+  require(q.ndim == 2 && q.shape[1] == (int64_t)heads * dk && out.ndim == 2 && out.shape[0] == M && out.shape[1] == (int64_t)heads * dv &&
+              q.dtype == pool.dtype && out.dtype == q.dtype && q.contiguous() && out.contiguous(),
+          "gated_attention: q/out/pool shapes or dtypes do not fit");
+  require(!sink.defined() || (sink.dtype == DType::F32 && sink.numel() == heads), "gated_attention: sink " + sink.describe() + " does not fit");
+  if (gate.mode) {
+    const int64_t need = gate.mode == 1 ? (int64_t)heads * dv : heads;
+    require((gate.mode == 1 || gate.mode == 2) && gate.proj.ndim == 2 && gate.proj.dtype == DType::F32 && gate.proj.contiguous() &&
+                gate.proj.shape[0] == M && gate.col >= 0 && gate.col + need <= gate.proj.shape[1],
+            "gated_attention: the gate's columns do not lie inside proj " + gate.proj.describe());
+  }
+  check_split_pool("gated_attention", pool, kv_heads, dk, dv, q.dtype);
+  took("[generic]");
+  int rc = KERNEL("gated_attention", ti_gated_attention_rows)(
+      code(q.dtype, "gated_attention"), q.data, pool.data, view.table, view.table_width, positions, slots,
+      sink.defined() ? (const float*)sink.data : nullptr, gate.mode ? (const float*)gate.proj.data + gate.col : nullptr,
+      gate.mode ? (int)gate.proj.shape[1] : 0, gate.mode, out.data, (int)M, heads, kv_heads, dk, dv, (int)pool.shape[2], scale, window,
+      (hipStream_t)launch_stream());
+  check("gated_attention", rc, "gated_attention");
+}
+
+void Ops::decay_scan(const Tensor& proj, const QkvColumns& cols, const Tensor& decay, const Tensor& state, const int* entry_meta,
+                     int n_entries, const Tensor& o, int heads, int dk, int dv) {
+  TIMED("decay_scan " + dims(proj) + " entries=" + std::to_string(n_entries));
+  require(proj.ndim == 2 && proj.dtype == DType::F32 && proj.contiguous(), "decay_scan: proj must be contiguous float32 [M, N]");
+  const int64_t per_slot = (int64_t)heads * dk * dv;
+  require(state.dtype == DType::F32 && state.contiguous() && state.ndim >= 2 && state.numel() == state.shape[0] * per_slot,
+          "decay_scan: state " + state.describe() + " does not fit [slots, " + std::to_string(heads) + ", " + std::to_string(dk * dv) + "]");
+  require(decay.dtype == DType::F32 && decay.numel() == heads, "decay_scan: decay " + decay.describe() + " must be float32 [heads]");
+  require(o.dtype == DType::F32 && o.contiguous() && o.ndim == 2 && o.shape[0] == proj.shape[0] && o.shape[1] == (int64_t)heads * dv,
+          "decay_scan: o " + o.describe() + " does not fit");
+  require(entry_meta != nullptr || n_entries == 0, "decay_scan: no entry records");
+  int rc = KERNEL("linear_attention", ti_decay_scan)((const float*)proj.data, (int)proj.shape[1], cols.q, cols.k, cols.v,
+                                                     (const float*)decay.data, (float*)state.data, (long)per_slot, entry_meta, n_entries,
+                                                     (float*)o.data, heads, dk, dv, (hipStream_t)launch_stream());
+  check("linear_attention", rc, "decay_scan");
+}
+
+void Ops::gated_row_norm(const Tensor& o, const Tensor& proj, int gate_col, const Tensor& w, float eps, const Tensor& out) {
+  TIMED("gated_row_norm " + dims(o));
+  require(o.ndim == 2 && o.dtype == DType::F32 && o.contiguous(), "gated_row_norm: o must be contiguous float32 [M, W]");
+  const int64_t M = o.shape[0], W = o.shape[1];
+  require(out.ndim == 2 && out.shape[0] == M && out.shape[1] == W && out.contiguous() && w.dtype == DType::F32 && w.numel() == W,
+          "gated_row_norm: out " + out.describe() + " or w " + w.describe() + " do not fit");
+  require(proj.ndim == 2 && proj.dtype == DType::F32 && proj.contiguous() && proj.shape[0] == M && gate_col >= 0 && gate_col + W <= proj.shape[1],
+          "gated_row_norm: the gate's columns do not lie inside proj " + proj.describe());
+  int rc = KERNEL("linear_attention", ti_gated_row_norm)(code(out.dtype, "gated_row_norm"), (const float*)o.data, (const float*)proj.data,
+                                                         (int)proj.shape[1], gate_col, (const float*)w.data, out.data, (int)M, (int)W, eps,
+                                                         (hipStream_t)launch_stream());
+  check("linear_attention", rc, "gated_row_norm");
+}
+
 // ------------------------------------------------- post-norm layers, short convolutions, differential attention, experts
 void Ops::norm_residual(const Tensor& x, const Tensor& y, const Tensor& gain, float eps, bool accumulate, const int* gather,
                         int n_gather, const Tensor* rounded) {
@@ -1308,6 +1452,11 @@ void Ops::diff_attention(const Tensor& q, const Tensor& pool, const CacheView& v
 
 void Ops::moe_route(const Tensor& h, const Tensor& router, const Tensor& ids, const Tensor& wts, int top, RouterScore score,
                     bool renormalize) {
+  moe_route(h, router, ids, wts, top, score, renormalize, RouterGroups());
+}
+
+void Ops::moe_route(const Tensor& h, const Tensor& router, const Tensor& ids, const Tensor& wts, int top, RouterScore score,
+                    bool renormalize, const RouterGroups& grouped) {
   TIMED("moe_route " + dims(h) + " experts=" + std::to_string(router.ndim == 2 ? router.shape[0] : 0));
   require(h.ndim == 2 && h.contiguous() && router.ndim == 2 && router.dtype == DType::F32 && router.contiguous() &&
               router.shape[1] == h.shape[1],
@@ -1316,9 +1465,13 @@ void Ops::moe_route(const Tensor& h, const Tensor& router, const Tensor& ids, co
   require(ids.dtype == DType::I32 && ids.contiguous() && ids.numel() == M * top && wts.dtype == DType::F32 && wts.contiguous() &&
               wts.numel() == M * top,
           "moe_route: ids and wts must be int32 / float32 [M, top]");
-  int rc = KERNEL("moe", ti_moe_route)(code(h.dtype, "moe_route"), h.data, (const float*)router.data, (int*)ids.data, (float*)wts.data,
-                                       (int)M, (int)h.shape[1], (int)router.shape[0], top, (int)score, renormalize ? 1 : 0,
-                                       (hipStream_t)launch_stream());
+  require(!grouped.correction.defined() || (grouped.correction.dtype == DType::F32 && grouped.correction.numel() == router.shape[0]),
+          "moe_route: correction " + grouped.correction.describe() + " must be float32 [experts]");
+  int rc = KERNEL("moe", ti_moe_route_grouped)(code(h.dtype, "moe_route"), h.data, (const float*)router.data,
+                                               grouped.correction.defined() ? (const float*)grouped.correction.data : nullptr,
+                                               (int*)ids.data, (float*)wts.data, (int)M, (int)h.shape[1], (int)router.shape[0], top,
+                                               (int)score, renormalize ? 1 : 0, grouped.groups, grouped.keep, grouped.weight_scale,
+                                               grouped.sum_floor, (hipStream_t)launch_stream());
   check("moe", rc, "moe_route");
 }
 

@@ -47,6 +47,17 @@
 //   block     "keep"        keeps a copy of the residual under a name for a later block of the step
 //   block     "mix_in"      x <- W [x; kept]: the residual and a kept stream through one learned matrix
 //
+//
+//   norm      "layernorm"   (x - mean) / sqrt(variance + eps) * w: a gain, no bias; also of a weighted sum of several streams
+//   block     "hyper"       the residual in several streams (hyper-connections): a sublayer reads norm(sum_s a_s x_s) and its output
+//                           y goes back as x_t <- sum_s B[s, t] x_s + c_t y; "hyper_spread" / "hyper_sum" open and close the streams
+//   mixer     "attention" with `sink` (a learned number a head in the softmax's denominator), `gate` (a sigmoid gate on the
+//                           heads' outputs, "entry" or "head"), `values_from_keys`, `v_mix` (values mixed with the first such
+//                           layer's), and a per-head norm beside keys and values of their own sizes
+//   mixer     "decay_attention" linear attention with a fixed decay per head, its state per request
+//   mixer     "sum"         two mixers side by side on the same input, added with fixed factors
+//   ffn       "glu" with `activation` "gelu_tanh"; "moe" with `correction`, `groups`, `weight_scale`, `sum_floor`
+//
 // A part gets every size and constant as a parameter and never looks at the model it sits in.
 #include <algorithm>
 #include <cmath>
@@ -113,6 +124,9 @@ std::string tensor_name(const Json& p, const char* key, const std::string& prefi
 
 void NormPart::forward_add(StepContext&, const Tensor&, const Tensor&, bool, const int*, int, const Tensor*) {
   throw EngineError(std::string("the norm '") + kind_name() + "' cannot write into the residual");
+}
+Rows NormPart::forward_mixed(StepContext&, const Tensor&, const Tensor&) {
+  throw EngineError(std::string("the norm '") + kind_name() + "' has no form for a sum of streams");
 }
 void MixerPart::forward_store(StepContext&, const Rows&, const Tensor&) {
   throw EngineError(std::string("the mixer '") + kind_name() + "' cannot write its output apart from the residual");
@@ -535,8 +549,33 @@ class Attention final : public MixerPart {
     // capped scores, a query temperature or values of another size than the keys: the kernels that serve these take
     // any sizes up to 256 and neither a per-head norm nor a rotation
     bias = p.has("bias") && p.at("bias").as_bool();
-    general = softcap > 0.f || temp_coef != 0.f || v_dim != head_dim || bias || (p.has("general") && p.at("general").as_bool());
-    if (general) {
+    // a sink, a gate, values from the keys or mixed with another layer's: the gated kernels (any sizes up to 256, a per-head norm too)
+    has_sink = p.has("sink") && p.at("sink").as_bool();
+    if (p.has("gate")) {
+      const std::string g = p.at("gate").as_string();
+      if (g != "entry" && g != "head") throw ConfigError("attention: gate '" + g + "' is not served (entry, head)");
+      gate_mode = g == "entry" ? 1 : 2;
+    }
+    values_from_keys = p.has("values_from_keys") && p.at("values_from_keys").as_bool();
+    if (p.has("v_mix")) {
+      const std::string vm = p.at("v_mix").as_string();
+      if (vm != "first" && vm != "mix") throw ConfigError("attention: v_mix '" + vm + "' is not served (first, mix)");
+      mix_mode = vm == "first" ? 1 : 2;
+    }
+    gated = has_sink || gate_mode != 0 || values_from_keys || mix_mode != 0;
+    if (gated) {
+      if (softcap > 0.f || temp_coef != 0.f || bias || (p.has("shares_kv") && p.at("shares_kv").as_bool()))
+        throw ConfigError("attention: a sink, a gate, values from the keys or mixed values go with neither capped scores, a query "
+                          "temperature, biases nor a shared cache");
+      if (values_from_keys && v_dim != head_dim) throw ConfigError("attention: values that are the keys have the keys' size");
+      if (values_from_keys && mix_mode) throw ConfigError("attention: values that are the keys are not mixed");
+    }
+    general = gated || softcap > 0.f || temp_coef != 0.f || v_dim != head_dim || bias || (p.has("general") && p.at("general").as_bool());
+    if (gated) {
+      if (head_dim < 1 || head_dim > 256 || v_dim < 1 || v_dim > 256)
+        throw ConfigError("attention: key size " + std::to_string(head_dim) + " / value size " + std::to_string(v_dim) +
+                          " are not served (up to 256)");
+    } else if (general) {
       if (head_dim < 1 || head_dim > 256 || v_dim < 1 || v_dim > 256)
         throw ConfigError("attention: key size " + std::to_string(head_dim) + " / value size " + std::to_string(v_dim) +
                           " are not served (up to 256)");
@@ -557,8 +596,14 @@ class Attention final : public MixerPart {
     if (!pos && p.has("pos")) pos = std::dynamic_pointer_cast<PositionPart>(build_part("pos", PartSpec::from_json(p.at("pos")), prefix));
     nq = (int64_t)heads * head_dim;
     nk = shares_kv ? 0 : (int64_t)kv_heads * head_dim;
-    nv = shares_kv ? 0 : (int64_t)kv_heads * v_dim;
+    nv = shares_kv || values_from_keys ? 0 : (int64_t)kv_heads * v_dim;
     no = (int64_t)heads * v_dim;
+    ng = gate_mode == 1 ? no : gate_mode == 2 ? heads : 0;
+    n_qn = tensor_name(p, "q_norm", prefix, "q_norm.weight");
+    n_kn = tensor_name(p, "k_norm", prefix, "k_norm.weight");
+    n_sink = tensor_name(p, "sink_tensor", prefix, "sink");
+    n_gate = tensor_name(p, "gate_tensor", prefix, "g");
+    n_vmix = tensor_name(p, "v_mix_tensor", prefix, "vmix");
     n_q = tensor_name(p, "q", prefix, "q_proj.weight");
     n_k = tensor_name(p, "k", prefix, "k_proj.weight");
     n_v = tensor_name(p, "v", prefix, "v_proj.weight");
@@ -591,11 +636,31 @@ class Attention final : public MixerPart {
     t.emplace_back(n_o, o);
     if (!shares_kv) {
       t.emplace_back(n_k, kv);
-      t.emplace_back(n_v, vv);
+      if (!values_from_keys) t.emplace_back(n_v, vv);
     }
     if (qk_norm) {
-      t.emplace_back(join(prefix, "q_norm.weight"), nw);
-      if (!shares_kv) t.emplace_back(join(prefix, "k_norm.weight"), nw);
+      t.emplace_back(n_qn, nw);
+      if (!shares_kv) t.emplace_back(n_kn, nw);
+    }
+    if (has_sink) {
+      TensorNeed sk;
+      sk.shape = {(int64_t)heads};
+      sk.role = TensorNeed::Vector;
+      sk.b = 1.0;
+      t.emplace_back(n_sink, sk);
+    }
+    if (gate_mode) {
+      TensorNeed g;
+      g.shape = {ng, hidden};
+      t.emplace_back(n_gate, g);
+    }
+    if (mix_mode) {      // one number; the layer whose values the others mix in holds it too, unused
+      TensorNeed lam;
+      lam.role = TensorNeed::Vector;
+      lam.init = "uniform";
+      lam.a = 0.2;
+      lam.b = 0.6;
+      t.emplace_back(n_vmix, lam);
     }
     if (bias) {
       // the biases of the projections: the tensor's name with ".b"
@@ -619,20 +684,25 @@ class Attention final : public MixerPart {
     }
     // q, k and v go straight into the fused matrix (the reference builds its fused copy beside the
     // originals and keeps both: /root/reference/src/inference.cu:154-169)
-    w_qkv = src.alloc(src.matrix_dtype, {nq + nk + nv, hidden});
+    w_qkv = src.alloc(src.matrix_dtype, {nq + nk + nv + ng, hidden});      // the gate's rows behind q, k and v: one product
     src.fill(n_q, w_qkv.rows(0, nq));
     if (!shares_kv) {
       src.fill(n_k, w_qkv.rows(nq, nk));
-      src.fill(n_v, w_qkv.rows(nq + nk, nv));
+      if (nv) src.fill(n_v, w_qkv.rows(nq + nk, nv));
     }
+    if (ng) src.fill(n_gate, w_qkv.rows(nq + nk + nv, ng));
     w_o = src.alloc(src.matrix_dtype, {hidden, no});
     src.fill(n_o, w_o);
     if (qk_norm) {
       TensorNeed nw;
       nw.shape = {head_dim};
       nw.role = TensorNeed::Vector;
-      q_norm_w = src.fetch(join(prefix, "q_norm.weight"), nw);
-      if (!shares_kv) k_norm_w = src.fetch(join(prefix, "k_norm.weight"), nw);
+      q_norm_w = src.fetch(n_qn, nw);
+      if (!shares_kv) k_norm_w = src.fetch(n_kn, nw);
+    }
+    for (const auto& kv : tensors()) {
+      if (has_sink && kv.first == n_sink) sink = src.fetch(kv.first, kv.second);
+      if (mix_mode && kv.first == n_vmix) mix_lambda = src.fetch(kv.first, kv.second);
     }
   }
   bool has_cache() const override { return true; }
@@ -742,12 +812,47 @@ class Attention final : public MixerPart {
       ctx.ops.attention_capped(q, pool, view, ctx.positions, ctx.slots, a, heads, kv_heads, head_dim, v_dim, scale, softcap, window);
     ctx.ops.linear(a, w_o, out, epi, epi == Ops::Add);
   }
+  // A sink, a gate, values from the keys or mixed with the first such layer's: one product with the stacked weight
+  // [q; k; v; gate] (32-bit sums), the preparation (per-head norms, rotation, the values' mixing, q out, k and v into the
+  // pages), attention with the sink in the denominator and the gate on its output, then the output projection.
+  void run_gated(StepContext& ctx, const Rows& h, const Tensor& out, Ops::Epilogue epi) {
+    const int64_t M = h.t.shape[0];
+    Tensor proj = ctx.buf("attn.qkv", DType::F32, {M, nq + nk + nv + ng});
+    ctx.ops.linear(h, w_qkv, proj, Ops::Store);
+    const auto bound = ctx.binding(this);
+    const Tensor pool = ctx.kv_pool(bound.first, bound.second);
+    const Ops::CacheView view = ctx.cache_view(bound.first);
+    Tensor q = ctx.buf("attn.q", ctx.act_dtype, {M, nq});
+    Ops::Rotation rot;
+    if (pos && !pos->fused(rot)) throw EngineError("attention: the position encoding '" + std::string(pos->kind_name()) + "' has no fused form");
+    Ops::QkvColumns cols;
+    cols.q = 0;
+    cols.k = (int)nq;
+    cols.v = values_from_keys ? -1 : (int)(nq + nk);
+    Ops::ValueMix mix;
+    mix.mode = mix_mode;
+    if (mix_mode) {
+      mix.kept = ctx.buf("attn.v_kept", DType::F32, {M, nv});
+      mix.lambda = mix_lambda;
+    }
+    ctx.ops.gated_qkv_prep(proj, cols, q_norm_w, k_norm_w, eps, rot, mix, ctx.positions, ctx.slots, view, pool, q, heads, kv_heads,
+                           head_dim, v_dim);
+    Tensor a = ctx.buf("attn.out", ctx.act_dtype, {M, no});
+    Ops::AttentionGate gate;
+    gate.mode = gate_mode;
+    gate.proj = proj;
+    gate.col = (int)(nq + nk + nv);
+    ctx.ops.gated_attention(q, pool, view, ctx.positions, ctx.slots, sink, gate, a, heads, kv_heads, head_dim, v_dim, scale, window);
+    ctx.ops.linear(a, w_o, out, epi, epi == Ops::Add);
+  }
   void forward_store(StepContext& ctx, const Rows& h, const Tensor& y) override {
     if (!general) return MixerPart::forward_store(ctx, h, y);
+    if (gated) return run_gated(ctx, h, y, Ops::Store);
     run_general(ctx, h, y, Ops::Store);
   }
 
   void forward(StepContext& ctx, const Rows& h, const Tensor& x) override {
+    if (gated) return run_gated(ctx, h, x, Ops::Add);
     if (general) return run_general(ctx, h, x, Ops::Add);
     const int64_t M = h.t.shape[0];
     const int64_t width = nq + 2 * nk;
@@ -807,9 +912,16 @@ class Attention final : public MixerPart {
   std::vector<std::pair<std::string, Tensor>> held() const override {
     return {{"w_qkv", w_qkv}, {"w_o", w_o}, {"q_norm_w", q_norm_w}, {"k_norm_w", k_norm_w}, {"b_qkv", b_qkv}};
   }
-  int64_t hidden = 0, nq = 0, nk = 0, nv = 0, no = 0;
+  int64_t hidden = 0, nq = 0, nk = 0, nv = 0, no = 0, ng = 0;
   int heads = 0, kv_heads = 0, head_dim = 0, v_dim = 0, window = 0, temp_every = 0;
   bool qk_norm = true, shares_kv = false, general = false, bias = false;
+  bool gated = false;             // any of the four below: the gated kernels run
+  bool has_sink = false;          // `sink`: exp(sink_h) joins the softmax's denominator (tensor `sink_tensor`, default prefix.sink)
+  int gate_mode = 0;              // `gate` "entry" (1) / "head" (2): the heads' outputs times sigmoid(W_g h) (tensor `gate_tensor`, prefix.g)
+  bool values_from_keys = false;  // `values_from_keys`: no value projection; a value is its key as projected
+  int mix_mode = 0;               // `v_mix` "first" (1): the values are kept for later layers; "mix" (2): v <- (1 - l) v + l kept
+  std::string n_qn, n_kn, n_sink, n_gate, n_vmix;
+  Tensor sink, mix_lambda;
   Tensor b_qkv;      // `bias`: the biases of q, k and v side by side, 32-bit
   float eps = 1e-6f, scale = 1.f, softcap = 0.f, temp_coef = 0.f;
   std::string n_q, n_k, n_v, n_o;
@@ -830,17 +942,25 @@ class PreNormBlock final : public BlockPart {
       if (kv.first == "norm2") norm2 = std::dynamic_pointer_cast<NormPart>(kv.second);
       if (kv.first == "ffn") ffn = std::dynamic_pointer_cast<FeedForwardPart>(kv.second);
     }
-    if (!norm1 || !mixer || !norm2 || !ffn) throw ConfigError("block 'pre_norm' needs norm1, mixer, norm2 and ffn parts");
+    if (!norm1 || !mixer) throw ConfigError("block 'pre_norm' needs norm1 and mixer parts (norm2 and ffn are optional)");
+    if ((ffn != nullptr) != (norm2 != nullptr)) throw ConfigError("block 'pre_norm': norm2 and ffn come together or not at all");
   }
   const char* kind_name() const override { return "pre_norm"; }
   bool reads_through_ops() const override { return true; }
-  std::vector<std::shared_ptr<Part>> children() const override { return {norm1, mixer, norm2, ffn}; }
-  std::vector<std::string> child_slots() const override { return {"norm1", "mixer", "norm2", "ffn"}; }
+  std::vector<std::shared_ptr<Part>> children() const override {
+    if (!ffn) return {norm1, mixer};
+    return {norm1, mixer, norm2, ffn};
+  }
+  std::vector<std::string> child_slots() const override {
+    if (!ffn) return {"norm1", "mixer"};
+    return {"norm1", "mixer", "norm2", "ffn"};
+  }
   void forward(StepContext& ctx, const Tensor& x) override {
     if (!norm1->reads_through_ops()) ctx.ops.flush();
     Rows h = norm1->forward(ctx, x, nullptr, 0, mixer->takes_lazy_norm() && norm1->can_be_lazy());
     if (!mixer->reads_through_ops()) ctx.ops.flush();
     mixer->forward(ctx, h, x);
+    if (!ffn) return;      // a layer without a feed-forward
     if (!norm2->reads_through_ops()) ctx.ops.flush();
     h = norm2->forward(ctx, x, nullptr, 0, ffn->takes_lazy_norm() && norm2->can_be_lazy());
     if (!ffn->reads_through_ops()) ctx.ops.flush();
@@ -1568,6 +1688,20 @@ class MoE final : public FeedForwardPart {
     scale_input = gated ? false : (!p.has("scale_input") || p.at("scale_input").as_bool());
     if (gated && p.has("scale_input") && p.at("scale_input").as_bool()) throw ConfigError("moe: gated experts take their weight on the output");
     n_router = tensor_name(p, "router", prefix, "router");
+    // a grouped router: a correction on the scores for the choice only, groups of neighbouring experts of which the best are
+    // kept, a factor on the weights, a floor under the sum they are divided by
+    corrected = p.has("correction") && p.at("correction").as_bool();
+    n_correction = tensor_name(p, "correction_tensor", prefix, "correction");
+    if (p.has("groups")) {
+      groups = (int)param_int(p.at("groups"), "count");
+      keep = (int)param_int(p.at("groups"), "keep");
+      if (groups < 1 || experts % groups || keep < 1 || keep > groups || (int64_t)keep * (experts / groups) < top)
+        throw ConfigError("moe: " + std::to_string(groups) + " groups of which " + std::to_string(keep) + " are kept do not fit " +
+                          std::to_string(experts) + " experts and top " + std::to_string(top));
+    }
+    weight_scale = p.has("weight_scale") ? (float)param_float(p, "weight_scale") : 1.f;
+    sum_floor = p.has("sum_floor") ? (float)param_float(p, "sum_floor") : 0.f;
+    if ((corrected || groups > 1) && score == Ops::SoftmaxChosen) throw ConfigError("moe: a correction or groups do not go with weights from the chosen logits");
     for (const auto& c : children)
       if (c.first == "shared") shared = std::dynamic_pointer_cast<FeedForwardPart>(c.second);
     if (!shared && p.has("shared")) {
@@ -1602,6 +1736,13 @@ class MoE final : public FeedForwardPart {
       t.emplace_back(expert_name(e, "down"), down);
     }
     t.emplace_back(n_router, router);
+    if (corrected) {
+      TensorNeed c;
+      c.shape = {(int64_t)experts};
+      c.role = TensorNeed::Vector;
+      c.b = 0.3;
+      t.emplace_back(n_correction, c);
+    }
     return t;
   }
   void load(WeightSource& src) override {
@@ -1619,13 +1760,29 @@ class MoE final : public FeedForwardPart {
     router.shape = {(int64_t)experts, hidden};
     router.role = TensorNeed::Vector;
     w_router = src.fetch(n_router, router);
+    if (corrected) {
+      TensorNeed c;
+      c.shape = {(int64_t)experts};
+      c.role = TensorNeed::Vector;
+      correction = src.fetch(n_correction, c);
+    }
   }
   void run(StepContext& ctx, const Rows& h, const Tensor& y, Ops::GatheredRows* left) {
     const Tensor& rows = h.materialize(ctx.ops);
     const int64_t M = rows.shape[0];
     Tensor ids = ctx.buf("moe.ids", DType::I32, {M, (int64_t)top});
     Tensor wts = ctx.buf("moe.wts", DType::F32, {M, (int64_t)top});
-    ctx.ops.moe_route(rows, w_router, ids, wts, top, score, renormalize);
+    if (corrected || groups > 1 || weight_scale != 1.f || sum_floor != 0.f) {
+      Ops::RouterGroups g;
+      g.correction = correction;
+      g.groups = groups;
+      g.keep = keep;
+      g.weight_scale = weight_scale;
+      g.sum_floor = sum_floor;
+      ctx.ops.moe_route(rows, w_router, ids, wts, top, score, renormalize, g);
+    } else {
+      ctx.ops.moe_route(rows, w_router, ids, wts, top, score, renormalize);
+    }
     if (gated) ctx.ops.moe_experts_gated(rows, ids, wts, w_up, w_down, y, experts, act_kind, limit, alpha, ctx.ws, left);
     else ctx.ops.moe_experts(rows, ids, wts, w_up, w_down, y, experts, scale_input, ctx.ws, left);
   }
@@ -1662,8 +1819,11 @@ class MoE final : public FeedForwardPart {
   Ops::GatedAct act_kind = Ops::Silu;
   float limit = 0.f, alpha = 1.702f;       // glu_clamped: g = min(g, limit), u = clamp(u, -limit, limit), g sigmoid(alpha g) (u + 1)
   std::shared_ptr<FeedForwardPart> shared; // `shared`: a feed-forward every token takes, added to the experts' sum
-  std::string n_router;
-  Tensor w_up, w_down, w_router;
+  std::string n_router, n_correction;
+  bool corrected = false;                  // `correction`: a vector added to the scores for the choice only (tensor prefix.correction)
+  int groups = 0, keep = 0;                // `groups` {count, keep}: only experts of the best `keep` of `count` groups can be chosen
+  float weight_scale = 1.f, sum_floor = 0.f;
+  Tensor w_up, w_down, w_router, correction;
 };
 
 // Dynamic Tanh in the place of a norm: y = tanh(alpha x) * w + b, alpha one learned number, w and b vectors; no mean and no
@@ -1707,7 +1867,8 @@ class DynamicTanh final : public NormPart {
   Tensor weight, alpha, bias;
 };
 
-// A gated feed-forward: down(act(gate h, up h)).  `activation` "silu": silu(g) u; "clamped" (`limit`, `alpha` default 1.702):
+// A gated feed-forward: down(act(gate h, up h)).  `activation` "silu": silu(g) u; "gelu_tanh": gelu(g) u with
+// gelu(g) = g / 2 (1 + tanh(sqrt(2 / pi) (g + 0.044715 g^3))); "clamped" (`limit`, `alpha` default 1.702):
 // g = min(g, limit), u = clamp(u, -limit, limit), g sigmoid(alpha g) (u + 1).  `bias`: every projection has a bias (the
 // tensor's name with ".b").  The first product leaves 32-bit sums of [gate | up] (one stacked weight), the activation is
 // taken in 32-bit and rounded once.  Tensor names: prefix + ".gate", ".up", ".down" unless the parameters give them.
@@ -1718,8 +1879,9 @@ class GatedFFN final : public FeedForwardPart {
     intermediate = param_int(p, "intermediate");
     if (hidden <= 0 || intermediate <= 0) throw ConfigError("glu feed-forward: sizes must be positive");
     const std::string act = p.has("activation") ? p.at("activation").as_string() : "silu";
-    if (act != "silu" && act != "clamped") throw ConfigError("glu feed-forward: activation '" + act + "' is not served (silu, clamped)");
-    kind = act == "clamped" ? Ops::ClampedGlu : Ops::Silu;
+    if (act != "silu" && act != "clamped" && act != "gelu_tanh")
+      throw ConfigError("glu feed-forward: activation '" + act + "' is not served (silu, clamped, gelu_tanh)");
+    kind = act == "clamped" ? Ops::ClampedGlu : act == "gelu_tanh" ? Ops::GeluTanh : Ops::Silu;
     if (kind == Ops::ClampedGlu) {
       limit = (float)param_float(p, "limit");
       alpha = p.has("alpha") ? (float)param_float(p, "alpha") : 1.702f;
@@ -2090,7 +2252,333 @@ class PostNormBlock final : public BlockPart {
   std::shared_ptr<FeedForwardPart> ffn;
 };
 
+// A layer norm with a gain and no bias: y = (x - mean(x)) / sqrt(mean((x - mean(x))^2) + eps) * w, in 32-bit, rounded once.
+// `tensor`: the weight's name in the checkpoint (default: prefix + ".weight").  It can norm 32-bit rows in place (an embedding's
+// rows) and take a weighted sum of several streams as its input without that sum being formed.
+class LayerNorm final : public NormPart {
+ public:
+  LayerNorm(const std::string& prefix, const Json& p) : NormPart(prefix) {
+    dim = param_int(p, "dim");
+    eps = (float)param_float(p, "eps");
+    name = tensor_name(p, "tensor", prefix, "weight");
+    if (dim <= 0 || dim > 16384) throw ConfigError("layernorm: a width of " + std::to_string(dim) + " is not served (1 to 16384)");
+  }
+  const char* kind_name() const override { return "layernorm"; }
+  bool reads_through_ops() const override { return true; }
+  std::vector<std::pair<std::string, TensorNeed>> tensors() const override {
+    TensorNeed n;
+    n.shape = {dim};
+    n.role = TensorNeed::Vector;
+    n.a = 1.0;
+    n.b = 0.1;
+    return {{name, n}};
+  }
+  void load(WeightSource& src) override { weight = src.fetch(name, tensors()[0].second); }
+  Rows forward(StepContext& ctx, const Tensor& x, const int* rows, int64_t n_rows, bool) override {
+    Rows r;
+    r.t = ctx.buf("norm.out", ctx.act_dtype, {rows ? n_rows : x.shape[0], dim});
+    ctx.ops.layernorm(x, weight, eps, r.t, rows, n_rows);
+    return r;
+  }
+  bool can_add() const override { return true; }
+  void forward_add(StepContext& ctx, const Tensor& y, const Tensor& x, bool accumulate, const int* gather, int n_gather,
+                   const Tensor* rounded) override {
+    if (accumulate || gather || n_gather > 1 || rounded) throw EngineError("layernorm: it norms 32-bit rows in place, nothing else");
+    ctx.ops.layernorm(y, weight, eps, x);
+  }
+  bool can_mix() const override { return true; }
+  Rows forward_mixed(StepContext& ctx, const Tensor& streams, const Tensor& coef) override {
+    Rows r;
+    r.t = ctx.buf("norm.out", ctx.act_dtype, {streams.shape[1], dim});
+    ctx.ops.layernorm_mixed(streams, coef, weight, eps, r.t);
+    return r;
+  }
+  std::vector<std::pair<std::string, Tensor>> held() const override { return {{"weight", weight}}; }
+  int64_t dim = 0;
+  float eps = 1e-6f;
+  std::string name;
+  Tensor weight;
+};
+
+// The residual in `streams` copies (hyper-connections).  "hyper_spread" makes every stream a copy of the residual as the
+// embedding left it; a "hyper" layer works on the streams; "hyper_sum" puts their sum back into the residual for the final
+// norm.  The streams of a step lie in the workspace under one name, f32 [streams, M, dim].
+static Tensor hyper_streams(StepContext& ctx, int64_t streams, int64_t M, int64_t dim) {
+  return ctx.buf("hyper.streams", DType::F32, {streams, M, dim});
+}
+class HyperSpreadBlock final : public BlockPart {
+ public:
+  HyperSpreadBlock(const std::string& prefix, const Json& p) : BlockPart(prefix), streams(param_int(p, "streams")), dim(param_int(p, "dim")) {}
+  const char* kind_name() const override { return "hyper_spread"; }
+  void forward(StepContext& ctx, const Tensor& x) override {
+    ctx.ops.flush();
+    ctx.ops.hyper_spread(x, hyper_streams(ctx, streams, x.shape[0], dim));
+  }
+  int64_t streams, dim;
+};
+class HyperSumBlock final : public BlockPart {
+ public:
+  HyperSumBlock(const std::string& prefix, const Json& p) : BlockPart(prefix), streams(param_int(p, "streams")), dim(param_int(p, "dim")) {}
+  const char* kind_name() const override { return "hyper_sum"; }
+  void forward(StepContext& ctx, const Tensor& x) override {
+    ctx.ops.flush();
+    ctx.ops.hyper_combine(hyper_streams(ctx, streams, x.shape[0], dim), Tensor(), x);
+  }
+  int64_t streams, dim;
+};
+
+// A layer on a residual of `streams` copies x_1 .. x_S.  Sublayer q (1: the mixer, 2: the feed-forward, which may be absent)
+// reads u = sum_s in_q[s] x_s through its norm, and its output y goes back into all streams at once:
+// x_t <- sum_s mix_q[s, t] x_s + out_q[t] y (mix indexed [from, to]).  Tensors: prefix + ".hc<q>.in" [S], ".hc<q>.out" [S],
+// ".hc<q>.mix" [S, S], held in 32-bit.  A norm that can take the weighted sum in does (no u is written); the sublayers write
+// apart from the residual.
+class HyperBlock final : public BlockPart {
+ public:
+  HyperBlock(const std::string& prefix, const Json& p, const PartChildren& c) : BlockPart(prefix) {
+    for (const auto& kv : c) {
+      if (kv.first == "norm1") norm1 = std::dynamic_pointer_cast<NormPart>(kv.second);
+      if (kv.first == "mixer") mixer = std::dynamic_pointer_cast<MixerPart>(kv.second);
+      if (kv.first == "norm2") norm2 = std::dynamic_pointer_cast<NormPart>(kv.second);
+      if (kv.first == "ffn") ffn = std::dynamic_pointer_cast<FeedForwardPart>(kv.second);
+    }
+    if (!norm1 || !mixer) throw ConfigError("block 'hyper' needs norm1 and mixer parts (norm2 and ffn are optional)");
+    if ((ffn != nullptr) != (norm2 != nullptr)) throw ConfigError("block 'hyper': norm2 and ffn come together or not at all");
+    if (!mixer->can_store() || (ffn && !ffn->can_store()))
+      throw ConfigError("block 'hyper': its mixer and feed-forward must be able to write their output apart from the residual");
+    streams = param_int(p, "streams");
+    dim = param_int(p, "dim");
+    if (streams < 1 || streams > 16) throw ConfigError("block 'hyper': " + std::to_string(streams) + " streams are not served (1 to 16)");
+  }
+  const char* kind_name() const override { return "hyper"; }
+  bool reads_through_ops() const override { return true; }
+  std::vector<std::shared_ptr<Part>> children() const override {
+    std::vector<std::shared_ptr<Part>> v = {norm1, mixer};
+    if (ffn) {
+      v.push_back(norm2);
+      v.push_back(ffn);
+    }
+    return v;
+  }
+  std::vector<std::string> child_slots() const override {
+    std::vector<std::string> v = {"norm1", "mixer"};
+    if (ffn) {
+      v.push_back("norm2");
+      v.push_back("ffn");
+    }
+    return v;
+  }
+  std::string name(int q, const char* t) const { return join(prefix, "hc" + std::to_string(q) + "." + t); }
+  std::vector<std::pair<std::string, TensorNeed>> tensors() const override {
+    std::vector<std::pair<std::string, TensorNeed>> t;
+    for (int q = 1; q <= (ffn ? 2 : 1); ++q) {
+      TensorNeed in, out, mix;
+      in.shape = out.shape = {streams};
+      mix.shape = {streams, streams};
+      in.role = out.role = mix.role = TensorNeed::Vector;
+      in.a = 1.0 / (double)streams;
+      in.b = 0.2;
+      out.a = 1.0;
+      out.b = 0.3;
+      mix.a = 1.0 / (double)streams;
+      mix.b = 0.3;
+      t.emplace_back(name(q, "in"), in);
+      t.emplace_back(name(q, "out"), out);
+      t.emplace_back(name(q, "mix"), mix);
+    }
+    return t;
+  }
+  void load(WeightSource& src) override {
+    const auto t = tensors();
+    for (int q = 0; q < (ffn ? 2 : 1); ++q) {
+      w_in[q] = src.fetch(t[3 * q].first, t[3 * q].second);
+      w_out[q] = src.fetch(t[3 * q + 1].first, t[3 * q + 1].second);
+      w_mix[q] = src.fetch(t[3 * q + 2].first, t[3 * q + 2].second);
+    }
+  }
+  Rows read(StepContext& ctx, NormPart& norm, const Tensor& xs, const Tensor& coef) {
+    if (norm.can_mix()) return norm.forward_mixed(ctx, xs, coef);
+    Tensor u = ctx.buf("hyper.u", DType::F32, {xs.shape[1], dim});
+    ctx.ops.hyper_combine(xs, coef, u);
+    return norm.forward(ctx, u);
+  }
+  void forward(StepContext& ctx, const Tensor& x) override {
+    const int64_t M = x.shape[0];
+    const Tensor xs = hyper_streams(ctx, streams, M, dim);
+    Tensor y = ctx.buf("hyper.y", DType::F32, {M, dim});
+    mixer->forward_store(ctx, read(ctx, *norm1, xs, w_in[0]), y);
+    ctx.ops.hyper_write(xs, w_mix[0], w_out[0], y);
+    if (!ffn) return;
+    ffn->forward_store(ctx, read(ctx, *norm2, xs, w_in[1]), y);
+    ctx.ops.hyper_write(xs, w_mix[1], w_out[1], y);
+  }
+  std::vector<std::pair<std::string, Tensor>> held() const override {
+    return {{"in1", w_in[0]}, {"out1", w_out[0]}, {"mix1", w_mix[0]}, {"in2", w_in[1]}, {"out2", w_out[1]}, {"mix2", w_mix[1]}};
+  }
+  std::shared_ptr<NormPart> norm1, norm2;
+  std::shared_ptr<MixerPart> mixer;
+  std::shared_ptr<FeedForwardPart> ffn;
+  int64_t streams = 1, dim = 0;
+  Tensor w_in[2], w_out[2], w_mix[2];
+};
+
+// Linear attention with a fixed decay per head.  q = silu(W_q h), k = silu(W_k h) (heads x head_dim), v = silu(W_v h)
+// (heads x v_head_dim); per head S_t = decay_h S_(t-1) + k_t v_t^T and o_t = S_t^T q_t, no other scale; the heads side by side
+// are divided by their root mean square over the whole row (eps), multiplied by the vector `norm` and by sigmoid(W_g h), and W_o
+// maps them back.  q, k, v and the gate come from one product with the stacked weight [q; k; v; g].  S (heads x head_dim x
+// v_head_dim) is per-request state in 32-bit, zero at admission; activations, state, outputs and the norm are 32-bit.
+// `decay`: the heads' factors.  Tensor names: prefix + ".q", ".k", ".v", ".g", ".o", ".norm".
+class DecayAttention final : public MixerPart {
+ public:
+  DecayAttention(const std::string& prefix, const Json& p) : MixerPart(prefix) {
+    hidden = param_int(p, "hidden");
+    heads = (int)param_int(p, "heads");
+    dk = (int)param_int(p, "head_dim");
+    dv = p.has("v_head_dim") ? (int)param_int(p, "v_head_dim") : dk;
+    eps = (float)param_float(p, "eps");
+    if (heads <= 0 || dk <= 0 || dv <= 0 || hidden <= 0) throw ConfigError("decay_attention: sizes must be positive");
+    if (dk > 256 || dv > 256) throw ConfigError("decay_attention: a state of " + std::to_string(dk) + " x " + std::to_string(dv) + " a head is not served (up to 256 x 256)");
+    const Json* d = p.find("decay");
+    if (!d || d->type() != Json::Array || (int)d->size() != heads) throw ConfigError("decay_attention: 'decay' must list one factor a head");
+    for (const Json& v : d->items()) {
+      if (!v.is_number()) throw ConfigError("decay_attention: 'decay' must hold numbers");
+      decay.push_back((float)v.as_double());
+    }
+    nq = (int64_t)heads * dk;
+    nv = (int64_t)heads * dv;
+    width = 2 * nq + 2 * nv;
+  }
+  const char* kind_name() const override { return "decay_attention"; }
+  bool takes_lazy_norm() const override { return true; }
+  bool reads_through_ops() const override { return true; }
+  bool can_store() const override { return true; }
+  std::string name(const char* t) const { return join(prefix, t); }
+  std::vector<std::pair<std::string, TensorNeed>> tensors() const override {
+    TensorNeed qk, v, o, nw;
+    qk.shape = {nq, hidden};
+    v.shape = {nv, hidden};
+    o.shape = {hidden, nv};
+    nw.shape = {nv};
+    nw.role = TensorNeed::Vector;
+    nw.a = 1.0;
+    nw.b = 0.1;
+    return {{name("q"), qk}, {name("k"), qk}, {name("v"), v}, {name("g"), v}, {name("o"), o}, {name("norm"), nw}};
+  }
+  void load(WeightSource& src) override {
+    w_in = src.alloc(src.matrix_dtype, {width, hidden});
+    src.fill(name("q"), w_in.rows(0, nq));
+    src.fill(name("k"), w_in.rows(nq, nq));
+    src.fill(name("v"), w_in.rows(2 * nq, nv));
+    src.fill(name("g"), w_in.rows(2 * nq + nv, nv));
+    const auto t = tensors();
+    w_o = src.fetch(t[4].first, t[4].second);
+    norm_w = src.fetch(t[5].first, t[5].second);
+    w_decay = src.alloc(DType::F32, {(int64_t)heads});
+    put_floats(w_decay, decay, src.to_host);
+  }
+  static void put_floats(const Tensor& dst, const std::vector<float>& values, bool on_host);
+  bool has_cache() const override { return true; }
+  CacheNeed cache_need() const override {
+    CacheNeed n;
+    n.kind = CacheNeed::State;
+    n.state_shape = {heads, (int64_t)dk * dv};
+    return n;
+  }
+  void run(StepContext& ctx, const Rows& h, const Tensor& out, Ops::Epilogue epi) {
+    const int64_t M = h.t.shape[0];
+    Tensor proj = ctx.buf("decay.proj", DType::F32, {M, width});
+    ctx.ops.linear(h, w_in, proj, Ops::Store);
+    const auto bound = ctx.binding(this);
+    const Tensor state = ctx.state(bound.first, bound.second);
+    Tensor o = ctx.buf("decay.o", DType::F32, {M, nv});
+    Ops::QkvColumns cols;
+    cols.q = 0;
+    cols.k = (int)nq;
+    cols.v = (int)(2 * nq);
+    ctx.ops.decay_scan(proj, cols, w_decay, state, ctx.entry_meta, (int)ctx.entries.size(), o, heads, dk, dv);
+    Tensor a = ctx.buf("decay.gated", ctx.act_dtype, {M, nv});
+    ctx.ops.gated_row_norm(o, proj, (int)(2 * nq + nv), norm_w, eps, a);
+    ctx.ops.linear(a, w_o, out, epi, epi == Ops::Add);
+  }
+  void forward(StepContext& ctx, const Rows& h, const Tensor& x) override { run(ctx, h, x, Ops::Add); }
+  void forward_store(StepContext& ctx, const Rows& h, const Tensor& y) override { run(ctx, h, y, Ops::Store); }
+  std::vector<std::pair<std::string, Tensor>> held() const override {
+    return {{"w_in", w_in}, {"w_o", w_o}, {"norm_w", norm_w}, {"decay", w_decay}};
+  }
+  int64_t hidden = 0, nq = 0, nv = 0, width = 0;
+  int heads = 0, dk = 0, dv = 0;
+  float eps = 1e-6f;
+  std::vector<float> decay;
+  Tensor w_in, w_o, norm_w, w_decay;
+};
+
+// Two mixers side by side on the same input: y = left_scale * left(h) + right_scale * right(h), added in 32-bit.  `left`,
+// `right`: the two mixers as parts ({"kind", "params", "name"}; the name follows this part's prefix); each keeps its own cache
+// or state.
+class SumMixer final : public MixerPart {
+ public:
+  SumMixer(const std::string& prefix, const Json& p, const PartChildren& children) : MixerPart(prefix) {
+    dim = param_int(p, "hidden");
+    left_scale = (float)param_float(p, "left_scale");
+    right_scale = (float)param_float(p, "right_scale");
+    for (const auto& c : children) {
+      if (c.first == "left") left = std::dynamic_pointer_cast<MixerPart>(c.second);
+      if (c.first == "right") right = std::dynamic_pointer_cast<MixerPart>(c.second);
+    }
+    auto build = [&](const char* key) {
+      const PartSpec sp = PartSpec::from_json(p.at(key));
+      return std::dynamic_pointer_cast<MixerPart>(build_part("mixer", sp, join(prefix, sp.name)));
+    };
+    if (!left && p.has("left")) left = build("left");
+    if (!right && p.has("right")) right = build("right");
+    if (!left || !right) throw ConfigError("mixer 'sum' needs a left and a right mixer");
+    if (!left->can_store() || !right->can_store()) throw ConfigError("mixer 'sum': both mixers must be able to write their output apart from the residual");
+  }
+  const char* kind_name() const override { return "sum"; }
+  bool can_store() const override { return true; }
+  bool reads_through_ops() const override { return left->reads_through_ops() && right->reads_through_ops(); }
+  std::vector<std::shared_ptr<Part>> children() const override { return {left, right}; }
+  std::vector<std::string> child_slots() const override { return {"left", "right"}; }
+  void load(WeightSource& src) override {
+    s_left = src.alloc(DType::F32, {dim});
+    s_right = src.alloc(DType::F32, {dim});
+    DecayAttention::put_floats(s_left, std::vector<float>((size_t)dim, left_scale), src.to_host);
+    DecayAttention::put_floats(s_right, std::vector<float>((size_t)dim, right_scale), src.to_host);
+  }
+  void run(StepContext& ctx, const Rows& h, const Tensor& x) {
+    const int64_t M = h.t.shape[0];
+    Tensor y1 = ctx.buf("sum.left", DType::F32, {M, dim}), y2 = ctx.buf("sum.right", DType::F32, {M, dim});
+    left->forward_store(ctx, h, y1);
+    right->forward_store(ctx, h, y2);
+    ctx.ops.scaled_add(x, y1, s_left, y2, s_right);
+  }
+  void forward(StepContext& ctx, const Rows& h, const Tensor& x) override { run(ctx, h, x); }
+  void forward_store(StepContext& ctx, const Rows& h, const Tensor& y) override {
+    ctx.ops.fill_zero(y.data, y.bytes());
+    run(ctx, h, y);
+  }
+  std::shared_ptr<MixerPart> left, right;
+  int64_t dim = 0;
+  float left_scale = 1.f, right_scale = 1.f;
+  Tensor s_left, s_right;      // the factors spread over a row: what the kernel that adds two scaled branches takes
+};
+
 void register_builtin_parts() {
+  register_part("norm", "layernorm", [](const std::string& prefix, const Json& p, const PartChildren&) {
+    return std::make_shared<LayerNorm>(prefix, p);
+  });
+  register_part("block", "hyper_spread",
+                [](const std::string& prefix, const Json& p, const PartChildren&) { return std::make_shared<HyperSpreadBlock>(prefix, p); });
+  register_part("block", "hyper_sum",
+                [](const std::string& prefix, const Json& p, const PartChildren&) { return std::make_shared<HyperSumBlock>(prefix, p); });
+  register_part("block", "hyper",
+                [](const std::string& prefix, const Json& p, const PartChildren& c) { return std::make_shared<HyperBlock>(prefix, p, c); },
+                {{"norm1", "norm"}, {"mixer", "mixer"}, {"norm2", "norm?"}, {"ffn", "ffn?"}});
+  register_part("mixer", "decay_attention", [](const std::string& prefix, const Json& p, const PartChildren&) {
+    return std::make_shared<DecayAttention>(prefix, p);
+  });
+  register_part("mixer", "sum", [](const std::string& prefix, const Json& p, const PartChildren& c) {
+    return std::make_shared<SumMixer>(prefix, p, c);
+  });
   register_part("pos", "rope_partial", [](const std::string& prefix, const Json& p, const PartChildren&) {
     return std::make_shared<RotaryPartial>(prefix, p);
   });
@@ -2159,7 +2647,7 @@ void register_builtin_parts() {
   });
   register_part("block", "pre_norm",
                 [](const std::string& prefix, const Json&, const PartChildren& c) { return std::make_shared<PreNormBlock>(prefix, c); },
-                {{"norm1", "norm"}, {"mixer", "mixer"}, {"norm2", "norm"}, {"ffn", "ffn"}});
+                {{"norm1", "norm"}, {"mixer", "mixer"}, {"norm2", "norm?"}, {"ffn", "ffn?"}});
 }
 
 // --------------------------------------------------------------------------------- foreign parts
@@ -2358,6 +2846,14 @@ float DiffAttention::lambda_of(const Tensor l[4], int dk, double diff, bool on_h
     s2 = std::fmaf(host[(size_t)2 * dk + d], host[(size_t)3 * dk + d], s2);
   }
   return std::exp(s1) - std::exp(s2) + (float)diff;
+}
+void DecayAttention::put_floats(const Tensor& dst, const std::vector<float>& values, bool on_host) {
+  if (on_host) {
+    memcpy(dst.data, values.data(), values.size() * 4);
+    return;
+  }
+  if (hipMemcpy(dst.data, values.data(), values.size() * 4, hipMemcpyHostToDevice) != hipSuccess)
+    throw KernelError("copying a part's constants to the device failed");
 }
 void RMSNorm::plus_one(const Tensor& w, const Tensor& out, bool on_host) {
   const size_t n = (size_t)w.numel();
