@@ -274,9 +274,9 @@ ModelSpec dubozen_spec(const Json& config) {
       mix.params.set("sink", true);
       mix.params.set("sink_tensor", at + ".sink");
       mix.params.set("gate", "entry");
+      mix.params.set("v_mix_tensor", at + ".vmix");
       if (m.at("v_mix").as_bool()) {
         mix.params.set("v_mix", first_mix_seen ? "mix" : "first");
-        mix.params.set("v_mix_tensor", at + ".vmix");
         first_mix_seen = true;
       }
     } else {

@@ -1255,6 +1255,63 @@ int ti_ops_call(void* ops_, const char* op_, const ti_tensor* t, int n_t, const 
     ops.gated_act(arg(0), arg(1), arg(2), (Ops::GatedAct)(int)num(0), (float)num(1), (float)num(2));
   } else if (op == "concat_round") {
     ops.concat_round(arg(0), arg(1), arg(2));
+  } else if (op == "layernorm") {
+    // x, w, out, rows (may be absent); eps
+    const bool rows = n_t > 3 && arg(3).defined();
+    ops.layernorm(arg(0), arg(1), (float)num(0), arg(2), rows ? iptr(3) : nullptr, rows ? arg(3).shape[0] : 0);
+  } else if (op == "layernorm_mixed") {
+    // streams [S, M, H], coef, w, out; eps
+    ops.layernorm_mixed(arg(0), arg(1), arg(2), (float)num(0), arg(3));
+  } else if (op == "hyper_combine") {
+    ops.hyper_combine(arg(0), arg(1), arg(2));      // streams, coef (may be absent), u
+  } else if (op == "hyper_spread") {
+    ops.hyper_spread(arg(0), arg(1));               // x, streams
+  } else if (op == "hyper_write") {
+    ops.hyper_write(arg(0), arg(1), arg(2), arg(3));      // streams, mix, back, y
+  } else if (op == "gated_qkv_prep") {
+    // proj, q_w, k_w, inv_freq, rope_table, positions, slots, table, pool, q_out, lambda, kept; eps, heads, kv_heads, dk, dv,
+    // columns of q, k, v (v < 0: the values are the keys), rotated entries, mix mode
+    Ops::Rotation r = rotation(3, 4);
+    r.dims = (int)num(8);
+    Ops::QkvColumns c;
+    c.q = (int)num(5);
+    c.k = (int)num(6);
+    c.v = (int)num(7);
+    Ops::ValueMix mix;
+    mix.mode = (int)num(9);
+    if (mix.mode) {
+      mix.lambda = arg(10);
+      mix.kept = arg(11);
+    }
+    ops.gated_qkv_prep(arg(0), c, arg(1), arg(2), (float)num(0), r, mix, iptr(5), iptr(6), view_of(7, arg(8)), arg(8), arg(9), (int)num(1),
+                       (int)num(2), (int)num(3), (int)num(4));
+  } else if (op == "gated_attention") {
+    // q, pool, table, positions, slots, sink, gate proj, out; heads, kv_heads, dk, dv, scale, window, gate column, gate mode
+    Ops::AttentionGate g;
+    g.mode = (int)num(7);
+    g.col = (int)num(6);
+    if (g.mode) g.proj = arg(6);
+    ops.gated_attention(arg(0), arg(1), view_of(2, arg(1)), iptr(3), iptr(4), arg(5), g, arg(7), (int)num(0), (int)num(1), (int)num(2),
+                        (int)num(3), (float)num(4), (int)num(5));
+  } else if (op == "decay_scan") {
+    // proj, decay, state, entries [R, 4], o; heads, dk, dv, columns of q, k, v
+    Ops::QkvColumns c;
+    c.q = (int)num(3);
+    c.k = (int)num(4);
+    c.v = (int)num(5);
+    ops.decay_scan(arg(0), c, arg(1), arg(2), iptr(3), (int)arg(3).shape[0], arg(4), (int)num(0), (int)num(1), (int)num(2));
+  } else if (op == "gated_row_norm") {
+    // o, proj, w, out; gate column, eps
+    ops.gated_row_norm(arg(0), arg(1), (int)num(0), arg(2), (float)num(1), arg(3));
+  } else if (op == "moe_route_grouped") {
+    // h, router, ids, wts, correction (may be absent); top, score, renormalize, groups, keep, weight scale, sum floor
+    Ops::RouterGroups g;
+    if (n_t > 4) g.correction = arg(4);
+    g.groups = (int)num(3);
+    g.keep = (int)num(4);
+    g.weight_scale = (float)num(5);
+    g.sum_floor = (float)num(6);
+    ops.moe_route(arg(0), arg(1), arg(2), arg(3), (int)num(0), (Ops::RouterScore)(int)num(1), num(2) != 0, g);
   } else if (op == "latent_prep") {
     // proj, norm_w, inv_freq, rope_table, positions, slots, table, pool; off_kv, eps, heads, dim, rot_dim, rank, rotated entries, mag
     Ops::Rotation r = rotation(2, 3);

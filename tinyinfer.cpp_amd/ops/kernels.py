@@ -100,7 +100,10 @@ _LIB_OF = {"embed": "core", "rmsnorm": "core", "rope_neox": "core", "rope_table"
            "scale": "residual", "short_conv": "diff_attention", "diff_qk_prep": "diff_attention", "diff_attention": "diff_attention",
            "moe_route": "moe", "moe_experts": "moe", "moe_experts_gated": "moe", "qkv_prep_write": "pointwise", "dyt": "pointwise",
            "gated_act": "pointwise", "concat_round": "pointwise", "latent_prep": "latent_attention",
-           "latent_attention": "latent_attention", "latent_transpose": "latent_attention"}
+           "latent_attention": "latent_attention", "latent_transpose": "latent_attention", "layernorm": "hyper",
+           "layernorm_mixed": "hyper", "hyper_combine": "hyper", "hyper_spread": "hyper", "hyper_write": "hyper",
+           "gated_qkv_prep": "gated_attention", "gated_attention": "gated_attention", "decay_scan": "linear_attention",
+           "gated_row_norm": "linear_attention", "moe_route_grouped": "moe"}
 
 
 class Ops:
@@ -416,7 +419,51 @@ class Ops:
     def gated_act(self, z, bias, out, activation="silu", limit=0.0, alpha=1.702):
         """z f32 [R, 2F] = [gate | up] (+ bias [2F]); "silu": silu(g) u; "clamped": g = min(g, limit), u = clamp(u, +-limit),
         g sigmoid(alpha g) (u + 1)."""
-        self._call("gated_act", [z, bias, out], [{"silu": 0, "clamped": 1}[activation], limit, alpha])
+        self._call("gated_act", [z, bias, out], [{"silu": 0, "clamped": 1, "gelu_tanh": 2}[activation], limit, alpha])
+
+    # ---- the layer norm, a residual in several streams, gated attention, linear attention with a fixed decay, a grouped router
+    def layernorm(self, x, w, eps, out, rows=None):
+        """out[r] = (x - mean) / sqrt(var + eps) * w of row rows[r] (or r); x float32; out may be x."""
+        self._call("layernorm", [x, w, out, rows], [eps])
+
+    def layernorm_mixed(self, streams, coef, w, eps, out):
+        """The same of sum_s coef[s] streams[s]; streams float32 [S, M, H]."""
+        self._call("layernorm_mixed", [streams, coef, w, out], [eps])
+
+    def hyper_combine(self, streams, coef, u):
+        self._call("hyper_combine", [streams, coef, u])
+
+    def hyper_spread(self, x, streams):
+        self._call("hyper_spread", [x, streams])
+
+    def hyper_write(self, streams, mix, back, y):
+        """streams[t] <- sum_s mix[s, t] streams[s] + back[t] y, every t at once."""
+        self._call("hyper_write", [streams, mix, back, y])
+
+    def gated_qkv_prep(self, proj, q_w, k_w, inv_freq, rope_table, positions, slots, table, pool, q_out, heads, kv_heads, dk, dv, columns,
+                       eps=1e-6, rot_dims=0, mix_mode=0, mix_lambda=None, kept=None):
+        """proj f32 [M, N] with q, k, v from `columns` on (v < 0: the values are the keys as projected); per-head norms (q_w, k_w
+        or None), rotation of the first rot_dims entries, mix_mode 1: the values also go to `kept`; 2: v <- (1 - l) v + l kept."""
+        self._call("gated_qkv_prep", [proj, q_w, k_w, inv_freq, rope_table, positions, slots, table, pool, q_out, mix_lambda, kept],
+                   [eps, heads, kv_heads, dk, dv] + list(columns) + [rot_dims, mix_mode])
+
+    def gated_attention(self, q, pool, table, positions, slots, sink, gate_proj, out, heads, kv_heads, dk, dv, scale, window=0, gate_col=0,
+                        gate_mode=0):
+        """Causal softmax attention with exp(sink[h]) in the denominator (sink None: none) and the output times sigmoid of the
+        gate columns of gate_proj (gate_mode 1: one an entry, 2: one a head, 0: none)."""
+        self._call("gated_attention", [q, pool, table, positions, slots, sink, gate_proj, out],
+                   [heads, kv_heads, dk, dv, scale, int(window or 0), gate_col, gate_mode])
+
+    def decay_scan(self, proj, decay, state, entries, o, heads, dk, dv, columns):
+        """entries int32 [R, 4] = (first row, tokens, -, state slot); S <- decay S + k v^T, o = S^T q on silu'd columns of proj."""
+        self._call("decay_scan", [proj, decay, state, entries, o], [heads, dk, dv] + list(columns))
+
+    def gated_row_norm(self, o, proj, gate_col, w, eps, out):
+        self._call("gated_row_norm", [o, proj, w, out], [gate_col, eps])
+
+    def moe_route_grouped(self, h, router, ids, wts, correction, top, groups=0, keep=0, weight_scale=1.0, sum_floor=0.0, renormalize=True):
+        """Sigmoid scores; `correction` joins them for the choice only; only experts of the `keep` best of `groups` groups can be chosen."""
+        self._call("moe_route_grouped", [h, router, ids, wts, correction], [top, 0, int(bool(renormalize)), groups, keep, weight_scale, sum_floor])
 
     def concat_round(self, a, b, out):
         self._call("concat_round", [a, b, out])

@@ -604,6 +604,7 @@ class Attention final : public MixerPart {
     n_sink = tensor_name(p, "sink_tensor", prefix, "sink");
     n_gate = tensor_name(p, "gate_tensor", prefix, "g");
     n_vmix = tensor_name(p, "v_mix_tensor", prefix, "vmix");
+    vmix_named = p.has("v_mix_tensor");
     n_q = tensor_name(p, "q", prefix, "q_proj.weight");
     n_k = tensor_name(p, "k", prefix, "k_proj.weight");
     n_v = tensor_name(p, "v", prefix, "v_proj.weight");
@@ -654,8 +655,9 @@ class Attention final : public MixerPart {
       g.shape = {ng, hidden};
       t.emplace_back(n_gate, g);
     }
-    if (mix_mode) {      // one number; the layer whose values the others mix in holds it too, unused
-      TensorNeed lam;
+    if (mix_mode || vmix_named) {      // one number; the layer whose values the others mix in holds it too, unused; a layer that
+      TensorNeed lam;                  // mixes nothing accepts one the checkpoint may carry
+      lam.optional = mix_mode == 0;
       lam.role = TensorNeed::Vector;
       lam.init = "uniform";
       lam.a = 0.2;
@@ -921,6 +923,7 @@ class Attention final : public MixerPart {
   bool values_from_keys = false;  // `values_from_keys`: no value projection; a value is its key as projected
   int mix_mode = 0;               // `v_mix` "first" (1): the values are kept for later layers; "mix" (2): v <- (1 - l) v + l kept
   std::string n_qn, n_kn, n_sink, n_gate, n_vmix;
+  bool vmix_named = false;
   Tensor sink, mix_lambda;
   Tensor b_qkv;      // `bias`: the biases of q, k and v side by side, 32-bit
   float eps = 1e-6f, scale = 1.f, softcap = 0.f, temp_coef = 0.f;
