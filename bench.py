@@ -35,6 +35,10 @@ model's own), a short convolution of four taps, keys visible inside blocks of
 `--mask-size` positions, and `--experts` experts of which a token takes `--top`, each
 sized so that a token's experts do the arithmetic of the model's dense feed-forward.
 
+`--design dubozen` does the same for a Dubozen decoder (a residual in several streams, attention
+with a sink, mixed values and gates, softmax attention beside linear attention with a fixed
+decay, a grouped router): `--mixers attention|parallel|alternate --ffn dense|moe --streams 2`.
+
 `--design nazorax` does the same for a Nazorax decoder: parallel layers behind a Dynamic
 Tanh, as mixers `--mixers attention` (biased, rotated attention with the model's heads
 under a window of `--window` positions), `latent` (latent attention with the model's
@@ -115,6 +119,27 @@ def nazorax_config(base, mixers, ffn, experts, top, window):
     L = base["num_hidden_layers"]
     return dict(architecture="Nazorax", width=H, vocab=base["vocab_size"], norm=dict(eps=1e-6), loop=dict(start=0, stop=L, times=1),
                 layers=[kinds[i % len(kinds)] for i in range(L)])
+
+
+def dubozen_config(base, mixers, ffn, experts, top, streams):
+    """A Dubozen config.json with the layer widths of the Qwen3 configuration `base`."""
+    H, F, hd = base["hidden_size"], base["intermediate_size"], base["head_dim"]
+    heads, kv = base["num_attention_heads"], base["num_key_value_heads"]
+    ff = max(64, (F // top) // 64 * 64)                  # top gated experts do what the gated dense one of F does
+    groups = 4 if experts % 4 == 0 and 2 * (experts // 4) >= top else 1
+    mlp = dict(kind="dense", ff=F) if ffn == "dense" else dict(kind="moe", expert=dict(ff=ff), router=dict(
+        experts=experts, top=top, scale=2.5, groups=dict(count=groups, keep=max(1, groups // 2))))
+    softmax = dict(heads=heads, kv_heads=kv, dim=hd, vdim=hd, scale=hd ** -0.5, rot=dict(base=1000000.0, dims=hd // 2))
+    attention = dict(type="attention", mixer=dict(softmax, v_mix=True), mlp=mlp)
+    decay = [1.0 - 2.0 ** (-5.0 - 3.0 * j / max(1, kv - 1)) for j in range(kv)]
+    parallel = dict(type="parallel", mixer=dict(left=softmax, right=dict(heads=kv, dim=hd, vdim=hd, decay=decay), left_scale=0.5, right_scale=0.5),
+                    mlp=mlp)
+    kinds = {"attention": [attention], "parallel": [parallel], "alternate": [attention, parallel]}[mixers]
+    cfg = dict(architecture="Dubozen", width=H, vocab=base["vocab_size"], norm=dict(eps=1e-6),
+               layers=[kinds[i % len(kinds)] for i in range(base["num_hidden_layers"])])
+    if streams:
+        cfg["streams"] = streams
+    return cfg
 
 
 MAX_SEQ = 4096            # context length a request may reach (more if --context asks for it)
@@ -432,15 +457,17 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--model", choices=sorted(MODELS), default="0.6b", help="whose layer sizes the model has")
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
-    ap.add_argument("--design", choices=["qwen3", "miterax", "mumasun", "nazorax"], default="qwen3",
-                    help="miterax / mumasun / nazorax: a decoder of that design with the layer widths of --model instead (see --mixers; --experts, --top, --mask-size; --ffn, --window)")
-    ap.add_argument("--experts", type=int, default=8, help="--design mumasun / nazorax: experts per layer")
-    ap.add_argument("--top", type=int, default=2, help="--design mumasun / nazorax: experts a token takes")
-    ap.add_argument("--ffn", choices=["dense", "moe"], default="moe", help="--design nazorax: the feed-forward of its layers")
+    ap.add_argument("--design", choices=["qwen3", "miterax", "mumasun", "nazorax", "dubozen"], default="qwen3",
+                    help="miterax / mumasun / nazorax / dubozen: a decoder of that design with the layer widths of --model instead (see --mixers; --experts, --top, --mask-size; --ffn, --window, --streams)")
+    ap.add_argument("--experts", type=int, default=8, help="--design mumasun / nazorax / dubozen: experts per layer")
+    ap.add_argument("--top", type=int, default=2, help="--design mumasun / nazorax / dubozen: experts a token takes")
+    ap.add_argument("--ffn", choices=["dense", "moe"], default="moe", help="--design nazorax / dubozen: the feed-forward of its layers")
+    ap.add_argument("--streams", type=int, default=2, help="--design dubozen: copies of the residual (0: one plain residual)")
     ap.add_argument("--window", type=int, default=1024, help="--design nazorax: positions an attention layer's window keeps")
     ap.add_argument("--mask-size", type=int, default=4096, help="--design mumasun: positions of a block of visible keys")
-    ap.add_argument("--mixers", choices=["attention", "mlstm", "latent", "alternate"], default="alternate",
-                    help="--design miterax (attention, mlstm, alternate) / nazorax (attention, latent, alternate): the mixer of its layers")
+    ap.add_argument("--mixers", choices=["attention", "mlstm", "latent", "parallel", "alternate"], default="alternate",
+                    help="--design miterax (attention, mlstm, alternate) / nazorax (attention, latent, alternate) / dubozen (attention, parallel, "
+                         "alternate): the mixer of its layers")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=2048, help="cached tokens each decoding request holds")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
@@ -485,6 +512,14 @@ def main() -> int:
         model_name = f"Nazorax ({args.mixers} mixers, {what}) at {NAMES[args.model]} sizes"
     elif args.mixers == "latent":
         ap.error("--mixers latent goes with --design nazorax")
+    if args.design == "dubozen":
+        if args.mixers in ("mlstm", "latent"):
+            ap.error("--design dubozen has the mixers attention, parallel and alternate")
+        cfg = dubozen_config(cfg, args.mixers, args.ffn, args.experts, args.top, args.streams)
+        what = "dense feed-forward" if args.ffn == "dense" else f"{args.top} of {args.experts} experts"
+        model_name = f"Dubozen ({args.mixers} mixers, {what}, {args.streams or 'no'} streams) at {NAMES[args.model]} sizes"
+    elif args.mixers == "parallel":
+        ap.error("--mixers parallel goes with --design dubozen")
     rng = np.random.default_rng(0)
     context, prefill_tokens = args.context, args.prefill_tokens
     max_seq = max(MAX_SEQ, context + args.warmup + args.steps + 64, prefill_tokens, args.cached + args.portion)

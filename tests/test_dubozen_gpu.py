@@ -543,6 +543,56 @@ def test_graphs_replay_the_bfloat16_kernels(folders):
     assert outs[0] == outs[1]
 
 
+def test_matrix_core_attention_takes_the_sink_where_it_finishes_a_column(tmp_path):
+    """bfloat16 at keys and values of 64: a long prompt whole (tiles, in pairs and one by one), then single tokens with every
+    context split over workgroups and not split.  Every way agrees with the row-wise kernels and with the plain model; with
+    the sinks taken out of the weights the logits move, so the agreement is not of models that ignore them."""
+    from tinyinfer_amd.engine import StepEntry
+    config = dm.CONFIGS["wide"]
+    weights = dm.draw_weights(config, seed=77)
+    for k in weights:
+        if k.endswith(".sink"):
+            weights[k] = weights[k] + 3.0                 # sinks as heavy as dozens of keys together ...
+        if k in ("l1.mix.o", "l2.mix.o"):
+            weights[k] = weights[k] * 6.0                 # ... in layers that weigh much in the residual
+    folder = dm.write_folder(str(tmp_path / "sinks"), config, 0, weights)
+    w = dm.as_float64(weights)
+    toks = random_tokens(420, config["vocab"], 5)
+    want = plain.forward(config, w, toks)
+    no_sink = dict(w)
+    for k in w:
+        if k.endswith(".sink"):
+            no_sink[k] = w[k] - 30.0
+    assert np.median(errors(plain.forward(config, no_sink, toks[:64]), want[:64])) > 0.15
+
+    def run(fast, splits=0, paired=None):
+        engine = build_engine(folder, "bfloat16", 448)
+        engine.ops.use_fast_attention = fast
+        engine.ops.force_decode_splits = splits
+        engine.ops.force_paired_tiles = paired
+        engine.ops.count_calls(True)
+        rows = [engine.step([StepEntry("x", toks[:400], list(range(400)))]).cpu().numpy()]
+        for t in toks[400:]:
+            rows.append(engine.step([StepEntry("x", [t], [0])]).cpu().numpy())
+        names = [r["name"] for r in engine.ops.timing_report()]
+        engine.ops.count_calls(False)
+        return np.concatenate(rows).astype(np.float64), names
+
+    slow, names = run(False)
+    assert any(n.startswith("gated_attention") and n.endswith("[generic]") for n in names)
+    assert not any(n.endswith("[mfma]") and n.startswith("gated_attention") for n in names)
+    ok, seen = within({"x": slow}, {"x": want}, "bfloat16")
+    assert ok, seen
+    for splits, paired in ((0, None), (4, True), (1, False)):
+        fast, names = run(True, splits, paired)
+        assert any(n.startswith("gated_attention") and n.endswith("[mfma]") for n in names), names
+        ok, seen = within({"x": fast}, {"x": want}, "bfloat16")
+        assert ok, (splits, paired, seen)
+        e = errors(fast, slow)
+        # a router's choice within rounding of a tie may fall the other way at a position or two
+        assert np.median(e) < 2e-2 and (e > 0.08).mean() <= 0.05, (splits, paired, float(np.median(e)), float(e.max()))
+
+
 def plain_greedy(config, w, prompt, n_new):
     """(generated ids, how many of them stand clear of a tie within rounding)."""
     toks, sure = list(prompt), 0

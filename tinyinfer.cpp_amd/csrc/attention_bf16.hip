@@ -387,6 +387,18 @@ struct QueryLoads {
 // others' load units are then free for keys and values from the start, and the preparation
 // runs while those are on their way.  It costs registers (one wavefront per SIMD): for launches
 // of at most one workgroup per compute unit, where the start of the kernel is most of its time.
+// A learned sink in the softmax's denominator: exp(sink[head]) joins the sum where a column is finished (no key, no value,
+// not scaled).  m, lt: the column's maximum (in units of log 2) and the sum of its weights; lt becomes the new denominator
+// and the factor on the column's unscaled outputs comes back.  sink null: nothing changes.
+__device__ __forceinline__ float sink_join(const float* __restrict__ sink, int head, float m, float& lt) {
+  if (!sink) return 1.f;
+  const float s = sink[head] * TI_LOG2E;
+  const float m_new = fmaxf(m, s);
+  const float f = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - m_new);
+  lt = fmaf(lt, f, __builtin_amdgcn_exp2f(s - m_new));
+  return f;
+}
+
 #define DEC_TABLE_LDS 1024     // entries of a block-table row that the decode kernel can hold in LDS
 template <int HD, bool PREP, bool SHARED = false>
 __global__ void __launch_bounds__(256)
@@ -394,7 +406,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool
                    int table_stride, const int* __restrict__ pos, const int* __restrict__ slot,
                    const int* __restrict__ rows, bf16_t* __restrict__ out, float* __restrict__ part_o,
                    float* __restrict__ part_ml, int n_head, int n_kv, int P, float scale, int window,
-                   int n_splits, QKPrep prep, float softcap = 0.f) {
+                   int n_splits, QKPrep prep, float softcap = 0.f, const float* __restrict__ sink = nullptr) {
   __shared__ float s_o[4][HD / 16][4][64];
   __shared__ float s_m[4][16], s_l[4][16];
   __shared__ __attribute__((aligned(16))) bf16_t s_kv[PREP ? 2 * HD : 2];   // the row's own key, then its value
@@ -564,7 +576,8 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool
     }
     const int dim = d * 16 + quad * 4;
     if (n_splits == 1) {
-      const float inv = 1.0f / lt;
+      float den = lt;
+      const float inv = sink_join(sink, head, mm, den) / den;
       Frag4 r;
 #pragma unroll
       for (int i = 0; i < 4; ++i) r.h[i] = f2bf(acc[i] * inv);
@@ -588,7 +601,8 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool
 template <int HD>
 __global__ void __launch_bounds__(HD < 64 ? 64 : HD)
 attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                  const int* __restrict__ rows, bf16_t* __restrict__ out, int n_head, int n_splits) {
+                  const int* __restrict__ rows, bf16_t* __restrict__ out, int n_head, int n_splits,
+                  const float* __restrict__ sink = nullptr) {
   const int ridx = blockIdx.x, head = blockIdx.y, d = threadIdx.x;
   if (d >= HD) return;
   const int m_row = rows ? rows[ridx] : ridx;
@@ -619,7 +633,8 @@ attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ pa
         lt = fmaf(ml[j].y, w, lt);
         acc = split_accumulate(acc, v[j], w);
       }
-    out[((size_t)m_row * n_head + head) * HD + d] = f2bf(acc * (1.0f / lt));
+    const float f = sink_join(sink, head, mm, lt);
+    out[((size_t)m_row * n_head + head) * HD + d] = f2bf(acc * (f / lt));
   };
   if (n_splits <= 8) {
     at_once(std::integral_constant<int, 8>{});
@@ -654,7 +669,8 @@ attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ pa
     lt = fmaf(ml.y, w, lt);
     acc = split_accumulate(acc, po[(size_t)s * HD], w);
   }
-  out[((size_t)m_row * n_head + head) * HD + d] = f2bf(acc * (1.0f / lt));
+  const float f = sink_join(sink, head, mm, lt);
+  out[((size_t)m_row * n_head + head) * HD + d] = f2bf(acc * (f / lt));
 }
 
 // ================================================================== prefill
@@ -665,7 +681,8 @@ template <int HD>
 __global__ void __launch_bounds__(512)
 attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool, const int* __restrict__ table,
                     int table_stride, const int* __restrict__ tiles, const int* __restrict__ entries,
-                    bf16_t* __restrict__ out, int n_head, int n_kv, int P, float scale, int window, float softcap = 0.f) {
+                    bf16_t* __restrict__ out, int n_head, int n_kv, int P, float scale, int window, float softcap = 0.f,
+                    const float* __restrict__ sink = nullptr) {
   const int entry = tiles[2 * blockIdx.x], first = tiles[2 * blockIdx.x + 1];
   const int row0 = entries[4 * entry], n_tok = entries[4 * entry + 1], start = entries[4 * entry + 2];
   const int head = blockIdx.y;
@@ -710,7 +727,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ poo
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
   if (!col_ok) return;
-  const float inv = 1.0f / l;
+  const float inv = sink_join(sink, head, mx, l) / l;
 #pragma unroll
   for (int d = 0; d < HD / 16; ++d) {
     Frag4 r;
@@ -797,7 +814,7 @@ attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
                         const int* __restrict__ table, int table_stride, const int* __restrict__ tiles,
                         int n_tiles, const int* __restrict__ entries, bf16_t* __restrict__ out, int n_head,
                         int n_kv, int P, float scale, int window, float* __restrict__ part_o = nullptr,
-                        float* __restrict__ part_ml = nullptr, float softcap = 0.f) {
+                        float* __restrict__ part_ml = nullptr, float softcap = 0.f, const float* __restrict__ sink = nullptr) {
   // gridDim.z > 1: the keys a tile sees are cut into gridDim.z runs of whole turns, workgroup z takes
   // run z and leaves its maxima, sums and unscaled outputs in part_ml [row][head][z] = (m, l) and
   // part_o [row][head][z][HD] for the kernel that merges them
@@ -1190,7 +1207,7 @@ attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
       if (h == 0 && first_val == 0) reinterpret_cast<float2*>(part_ml)[at] = make_float2(m_all, lt);
       return;
     }
-    const float inv = 1.0f / lt;
+    const float inv = sink_join(sink, head, m_all, lt) / lt;
     bf16_t* dst = out + ((size_t)row * n_head + head) * HD;
 #pragma unroll
     for (int j = 0; j < n_val; j += 4) {
@@ -1314,6 +1331,10 @@ static int g_decode_shared_query = 1;
 // The soft cap of the call under way: the entry points whose names end in `_capped_bf16` set it around a call of
 // the plain ones, which hand it to their kernels (0: none).
 static thread_local float g_softcap = 0.f;
+// The sinks of the call under way (float [n_head] in device memory, or null): `ti_attention_bf16_sink` sets them for the calling
+// thread's next calls, which hand them to the kernels that finish a column.
+static thread_local const float* g_sink = nullptr;
+extern "C" void ti_attention_bf16_sink(const float* sink) { g_sink = sink; }
 
 template <bool PREP>
 static int launch_decode(const void* q, const void* pool, const int* table, int table_stride, const int* pos,
@@ -1335,16 +1356,16 @@ static int launch_decode(const void* q, const void* pool, const int* table, int 
     if (shared)                                                                                            \
       attn_decode_kernel<H, PREP, PREP><<<grid, 256, 0, stream>>>(                                         \
           (const bf16_t*)q, (const bf16_t*)pool, table, table_stride, pos, slot, rows, (bf16_t*)out,        \
-          part_o, part_ml, n_head, n_kv, page_size, scale, window, n_splits, prep, g_softcap);              \
+          part_o, part_ml, n_head, n_kv, page_size, scale, window, n_splits, prep, g_softcap, g_sink);      \
     else                                                                                                   \
       attn_decode_kernel<H, PREP><<<grid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)pool, table,   \
                                                             table_stride, pos, slot, rows, (bf16_t*)out,    \
                                                             part_o, part_ml, n_head, n_kv, page_size,       \
-                                                            scale, window, n_splits, prep, g_softcap);      \
+                                                            scale, window, n_splits, prep, g_softcap, g_sink); \
     if (n_splits > 1)                                                                                       \
       attn_merge_kernel<H><<<dim3(n_rows, n_head), (H < 64 ? 64 : H), 0, stream>>>(part_o, part_ml, rows,   \
                                                                                   (bf16_t*)out, n_head,    \
-                                                                                  n_splits);               \
+                                                                                  n_splits, g_sink);       \
     break;
   switch (hd) {
     TI_DEC(64) TI_DEC(128)
@@ -1353,10 +1374,10 @@ static int launch_decode(const void* q, const void* pool, const int* table, int 
         attn_decode_kernel<32, false><<<grid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)pool, table,
                                                                 table_stride, pos, slot, rows, (bf16_t*)out,
                                                                 part_o, part_ml, n_head, n_kv, page_size, scale,
-                                                                window, n_splits, prep, g_softcap);
+                                                                window, n_splits, prep, g_softcap, g_sink);
         if (n_splits > 1)
           attn_merge_kernel<32><<<dim3(n_rows, n_head), 64, 0, stream>>>(part_o, part_ml, rows, (bf16_t*)out,
-                                                                         n_head, n_splits);
+                                                                         n_head, n_splits, g_sink);
       }
       break;
   }
@@ -1446,7 +1467,7 @@ extern "C" int ti_attention_prefill_bf16(const void* q, const void* pool, const 
   attn_prefill_lds_kernel<H, G><<<grid, 256 * G, lds, stream>>>((const bf16_t*)q, (const bf16_t*)pool, table,   \
                                                                 table_stride, tiles, n_tiles, entries,          \
                                                                 (bf16_t*)out, n_head, n_kv, page_size, scale,   \
-                                                                window, nullptr, nullptr, g_softcap)
+                                                                window, nullptr, nullptr, g_softcap, g_sink)
     if (hd == 128 && groups == 2) TI_PLDS(128, 2);
     else if (hd == 128) TI_PLDS(128, 1);
     else if (groups == 2) TI_PLDS(64, 2);
@@ -1459,7 +1480,7 @@ extern "C" int ti_attention_prefill_bf16(const void* q, const void* pool, const 
   case H:                                                                                                  \
     attn_prefill_kernel<H><<<grid, 512, 0, stream>>>((const bf16_t*)q, (const bf16_t*)pool, table,          \
                                                      table_stride, tiles, entries, (bf16_t*)out, n_head,    \
-                                                     n_kv, page_size, scale, window, g_softcap);            \
+                                                     n_kv, page_size, scale, window, g_softcap, g_sink);    \
     break;
   switch (hd) {
     TI_PRE(32) TI_PRE(64) TI_PRE(128)
@@ -1512,7 +1533,7 @@ extern "C" int ti_attention_prefill_paired_bf16(const void* q, const void* pool,
 #define TI_GO(H, PAIRED)                                                                                          \
   attn_prefill_lds_kernel<H, NG, NW, ST, PAIRED, CB><<<grid, 64 * NW * NG, lds, stream>>>(                            \
       (const bf16_t*)q, (const bf16_t*)pool, table, table_stride, tiles, n_tiles, entries, (bf16_t*)out, n_head, \
-      n_kv, page_size, scale, window, part_o, part_ml, g_softcap)
+      n_kv, page_size, scale, window, part_o, part_ml, g_softcap, g_sink)
   if (hd == 128 && paired) TI_GO(128, true);
   else if (hd == 128) TI_GO(128, false);
   else if (paired) TI_GO(64, true);
@@ -1522,10 +1543,10 @@ extern "C" int ti_attention_prefill_paired_bf16(const void* q, const void* pool,
     // every row of the step has its runs (rows of single tokens too: theirs are not read by anyone)
     if (hd == 128)
       attn_merge_kernel<128><<<dim3(n_rows, n_head), 128, 0, stream>>>(part_o, part_ml, nullptr, (bf16_t*)out, n_head,
-                                                                     n_splits);
+                                                                     n_splits, g_sink);
     else
       attn_merge_kernel<64><<<dim3(n_rows, n_head), 64, 0, stream>>>(part_o, part_ml, nullptr, (bf16_t*)out, n_head,
-                                                                   n_splits);
+                                                                   n_splits, g_sink);
   }
   TI_LAUNCH_CHECK();
   return 0;

@@ -58,7 +58,7 @@ ONLY_FOR = {"pointwise": ("Miterax", "Nazorax", "Dubozen"), "recurrent": ("Miter
             "latent_attention": ("Nazorax",), "latent_attention_bf16": ("Nazorax",), "hyper": ("Dubozen",),
             "gated_attention": ("Dubozen",), "linear_attention": ("Dubozen",)}
 # ... and libraries that a named architecture never calls into
-NOT_FOR = {"attention_generic": ("Mumasun", "Dubozen"), "attention_bf16": ("Mumasun", "Dubozen")}
+NOT_FOR = {"attention_generic": ("Mumasun", "Dubozen"), "attention_bf16": ("Mumasun",)}
 
 
 def libraries_for(dtype: str, architecture: str = None) -> List[str]:

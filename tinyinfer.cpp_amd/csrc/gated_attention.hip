@@ -154,6 +154,31 @@ extern "C" int ti_gated_qkv_prep(int dtype, const float* proj, int ld, int off_q
   return 0;
 }
 
+// The gate on its own, behind attention kernels that do not take it in: a[m, h dv + d] *= sigmoid(gate[m, h dv + d] or gate[m, h])
+template <typename T>
+__global__ void sigmoid_gate_kernel(T* __restrict__ a, const float* __restrict__ gate, int gate_ld, int gate_mode, long n, int W, int dv) {
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+    const long m = i / W;
+    const int c = (int)(i % W);
+    const float z = gate[m * gate_ld + (gate_mode == 1 ? c : c / dv)];
+    st<T>(a + i, ld<T>(a + i) * (1.0f / (1.0f + expf(-z))));
+  }
+}
+
+extern "C" int ti_sigmoid_gate(int dtype, void* a, const float* gate, int gate_ld, int gate_mode, int M, int n_head, int dv,
+                               hipStream_t stream) {
+  TI_REQUIRE(M >= 0 && n_head > 0 && dv > 0 && gate && ((gate_mode == 1 && gate_ld >= n_head * dv) || (gate_mode == 2 && gate_ld >= n_head)),
+             "sigmoid_gate: bad sizes M=%d heads=%d dv=%d gate mode %d in rows of %d", M, n_head, dv, gate_mode, gate_ld);
+  if (M == 0) return 0;
+  const long n = (long)M * n_head * dv;
+  const unsigned blocks = (unsigned)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
+  if (dtype == TI_F32) sigmoid_gate_kernel<float><<<blocks, 256, 0, stream>>>((float*)a, gate, gate_ld, gate_mode, n, n_head * dv, dv);
+  else if (dtype == TI_BF16) sigmoid_gate_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)a, gate, gate_ld, gate_mode, n, n_head * dv, dv);
+  else TI_REQUIRE(false, "sigmoid_gate: unknown dtype %d", dtype);
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
 // ------------------------------------------------------------------------------------------------
 // A workgroup per (row, head): sixteen groups of sixteen lanes, group g the keys at positions g, g + 16, ... with a running
 // softmax each, merged in a fixed order (a key's group depends on its position alone, so every cut of the same tokens takes

@@ -191,6 +191,10 @@ int ti_mlstm_scan_chunked(const float* proj, int ld, int off_q, int off_k, int o
 int ti_gated_head_norm(int out_dtype, const float* o, const float* gate, int ld, int off_g, const float* w, void* out,
                        int M, int heads, int dv, float eps, hipStream_t stream);
 
+// libti_attention_bf16: sinks (float [n_head] in device memory, null: none) for the calling thread's next calls of the
+// matrix-core attention entry points: exp(sink[head]) joins the softmax's denominator where a column is finished
+void ti_attention_bf16_sink(const float* sink);
+
 // ---- libti_hyper: the layer norm, and a residual kept in several streams
 // out[r] = layernorm(sum_s coef[s] x_s[rows ? rows[r] : r]) * w (mean and variance, no bias), in `out_dtype`; the streams lie
 // stream_stride floats apart; coef null: the first stream alone.  out may be x (float32, one stream).  H up to 16384
@@ -214,6 +218,8 @@ int ti_gated_qkv_prep(int dtype, const float* proj, int ld, int off_q, int off_k
                       int mix_mode, const float* mix_lambda, float* v_kept, const int* pos, const int* slot, const int* table,
                       int table_stride, void* pool, void* q_out, int M, int n_head, int n_kv, int dk, int dv, int page_size,
                       hipStream_t stream);
+// a (T [M, n_head dv]) *= sigmoid(gate), gate f32 rows of gate_ld floats: entry h dv + d (gate_mode 1) or h (gate_mode 2)
+int ti_sigmoid_gate(int dtype, void* a, const float* gate, int gate_ld, int gate_mode, int M, int n_head, int dv, hipStream_t stream);
 // causal softmax attention of every row over such pages; sink f32 [n_head] (null: none) joins the denominator; gate (null:
 // none) f32 rows of gate_ld floats, the output times sigmoid of entry h dv + d (gate_mode 1) or h (gate_mode 2)
 int ti_gated_attention_rows(int dtype, const void* q, const void* pool, const int* table, int table_stride, const int* pos,

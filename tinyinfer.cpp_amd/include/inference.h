@@ -322,8 +322,11 @@ class Ops {
   void attention_rows(const Tensor& q, const Tensor& pool, const CacheView& view, const int* positions, const int* slots,
                       const Tensor& out, int heads, int kv_heads, int head_dim, float scale, int window);
   // softcap > 0: scores are capped, s <- softcap tanh(s / softcap), before the softmax
-  void attention(const AttentionWork& work, Workspace& ws, const CacheView& view, const Tensor& q, const Tensor& pool,
-                 const Tensor& out, int heads, int kv_heads, int head_dim, float scale, int window, float softcap = 0.f);
+  // sink (f32 [heads] in device memory, or null): exp(sink[h]) joins the softmax's denominator; only the matrix-core kernels take
+  // it: with a sink the call returns false, and nothing has run, where they do not serve the sizes
+  bool attention(const AttentionWork& work, Workspace& ws, const CacheView& view, const Tensor& q, const Tensor& pool,
+                 const Tensor& out, int heads, int kv_heads, int head_dim, float scale, int window, float softcap = 0.f,
+                 const float* sink = nullptr);
   bool attention_from_projections(const AttentionWork& work, Workspace& ws, const CacheView& view, const Tensor& qkv,
                                   const float* q_w, const float* k_w, float eps, const Rotation& rot, const Tensor& pool,
                                   bool write_kv, const Tensor& out, int heads, int kv_heads, int head_dim, float scale,
@@ -415,9 +418,10 @@ class Ops {
   // causal softmax attention over such pages with a sink (f32 [heads], undefined: none) in the denominator and a sigmoid gate on
   // the output read from proj's columns from gate_col on: gate_mode 1 one number an output entry, 2 one a head (0: no gate)
   struct AttentionGate { Tensor proj; int col = 0, mode = 0; };
+  // work, ws: the step's lists; with them, bfloat16, dk = dv and sizes the matrix-core kernels take, those run (the gate behind them)
   void gated_attention(const Tensor& q, const Tensor& pool, const CacheView& view, const int* positions, const int* slots,
                        const Tensor& sink, const AttentionGate& gate, const Tensor& out, int heads, int kv_heads, int dk, int dv,
-                       float scale, int window);
+                       float scale, int window, const AttentionWork* work = nullptr, Workspace* ws = nullptr);
   // Linear attention with a fixed decay per head over each entry's tokens, from and into its state slot: S <- decay_h S + k v^T,
   // o = S^T q with q, k, v = silu of proj's columns; decay f32 [heads]; state f32 [slots][heads][dk dv]; o f32 [M, heads dv]
   void decay_scan(const Tensor& proj, const QkvColumns& cols, const Tensor& decay, const Tensor& state, const int* entry_meta,

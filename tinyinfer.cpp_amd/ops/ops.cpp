@@ -789,9 +789,27 @@ bool Ops::attention_from_projections(const AttentionWork& work, Workspace& ws, c
   return true;
 }
 
-void Ops::attention(const AttentionWork& work, Workspace& ws, const CacheView& view, const Tensor& q, const Tensor& pool,
-                    const Tensor& out, int heads, int kv_heads, int head_dim, float scale, int window, float softcap) {
+namespace {
+// the sinks of the matrix-core attention calls made while this lives
+struct SinkScope {
+  explicit SinkScope(const float* sink) : set(sink != nullptr) {
+    if (set) KERNEL("attention_bf16", ti_attention_bf16_sink)(sink);
+  }
+  ~SinkScope() {
+    if (set) KERNEL("attention_bf16", ti_attention_bf16_sink)(nullptr);
+  }
+  bool set;
+};
+}  // namespace
+
+bool Ops::attention(const AttentionWork& work, Workspace& ws, const CacheView& view, const Tensor& q, const Tensor& pool,
+                    const Tensor& out, int heads, int kv_heads, int head_dim, float scale, int window, float softcap,
+                    const float* sink) {
+  if (sink && !(q.dtype == DType::BF16 && use.fast_attention && kernel_library_available("attention_bf16") &&
+                (head_dim == 32 || head_dim == 64 || head_dim == 128) && pool.ndim == 4 && pool.shape[2] % 16 == 0))
+    return false;
   TunedScope tuned(*this, "attention_bf16");
+  SinkScope sinks(sink);
   TIMED("attention rows=" + std::to_string(work.M) + (work.decode_only ? " decode" : " tiles=" + std::to_string(work.n_tiles) + " single=" + std::to_string(work.n_decode_rows)) + " context<=" + std::to_string(work.max_context));
   bool done = false;
   if (q.dtype == DType::BF16 && use.fast_attention && kernel_library_available("attention_bf16")) {
@@ -850,10 +868,12 @@ void Ops::attention(const AttentionWork& work, Workspace& ws, const CacheView& v
     }
   }
   took(done ? "[mfma]" : "[generic]");
+  if (!done && sink) throw KernelError("attention: the matrix-core kernels refused sizes they were asked about, with a sink to join");
   if (!done && softcap > 0.f)
     attention_capped(q, pool, view, work.positions, work.slots, out, heads, kv_heads, head_dim, head_dim, scale, softcap, window);
   else if (!done)
     attention_rows(q, pool, view, work.positions, work.slots, out, heads, kv_heads, head_dim, scale, window);
+  return true;
 }
 
 // ------------------------------------------------- layers beyond the pre-norm transformer block
@@ -1257,7 +1277,7 @@ void Ops::gated_qkv_prep(const Tensor& proj, const QkvColumns& cols, const Tenso
 
 void Ops::gated_attention(const Tensor& q, const Tensor& pool, const CacheView& view, const int* positions, const int* slots,
                           const Tensor& sink, const AttentionGate& gate, const Tensor& out, int heads, int kv_heads, int dk, int dv,
-                          float scale, int window) {
+                          float scale, int window, const AttentionWork* work, Workspace* ws) {
   TIMED("gated_attention " + dims(q) + (sink.defined() ? " sink" : "") + (gate.mode ? " gate" + std::to_string(gate.mode) : ""));
   const int64_t M = q.shape[0];
   require(q.ndim == 2 && q.shape[1] == (int64_t)heads * dk && out.ndim == 2 && out.shape[0] == M && out.shape[1] == (int64_t)heads * dv &&
@@ -1271,6 +1291,19 @@ void Ops::gated_attention(const Tensor& q, const Tensor& pool, const CacheView& 
             "gated_attention: the gate's columns do not lie inside proj " + gate.proj.describe());
   }
   check_split_pool("gated_attention", pool, kv_heads, dk, dv, q.dtype);
+  const float* gate_ptr = gate.mode ? (const float*)gate.proj.data + gate.col : nullptr;
+  if (work && ws && dk == dv && q.dtype == DType::BF16 && use.fast_attention && kernel_library_available("attention_bf16") &&
+      (dk == 32 || dk == 64 || dk == 128) && pool.shape[2] % 16 == 0) {
+    // the matrix-core kernels of plain attention, the sink joining where they finish a column; the gate behind them
+    attention(*work, *ws, view, q, pool, out, heads, kv_heads, dk, scale, window, 0.f, sink.defined() ? (const float*)sink.data : nullptr);
+    if (gate.mode) {
+      int rc = KERNEL("gated_attention", ti_sigmoid_gate)(code(out.dtype, "gated_attention"), out.data, gate_ptr, (int)gate.proj.shape[1],
+                                                          gate.mode, (int)M, heads, dv, (hipStream_t)launch_stream());
+      check("gated_attention", rc, "gated_attention(gate)");
+    }
+    took("[mfma]");
+    return;
+  }
   took("[generic]");
   int rc = KERNEL("gated_attention", ti_gated_attention_rows)(
       code(q.dtype, "gated_attention"), q.data, pool.data, view.table, view.table_width, positions, slots,

@@ -844,7 +844,9 @@ class Attention final : public MixerPart {
     gate.mode = gate_mode;
     gate.proj = proj;
     gate.col = (int)(nq + nk + nv);
-    ctx.ops.gated_attention(q, pool, view, ctx.positions, ctx.slots, sink, gate, a, heads, kv_heads, head_dim, v_dim, scale, window);
+    const AttentionWork w = work(ctx);
+    ctx.ops.gated_attention(q, pool, view, ctx.positions, ctx.slots, sink, gate, a, heads, kv_heads, head_dim, v_dim, scale, window,
+                            ctx.plan ? &w : nullptr, &ctx.ws);
     ctx.ops.linear(a, w_o, out, epi, epi == Ops::Add);
   }
   void forward_store(StepContext& ctx, const Rows& h, const Tensor& y) override {
