@@ -266,6 +266,17 @@ def test_decayed_linear_attention(ops, heads, dk, dv):
     state[0].zero_()                                          # the slot goes to the next request
     again = run([1] * 5 + [T - 5], 0)
     assert np.array_equal(again, whole)
+    # the tokens in chunks that run side by side, the state carried from chunk to chunk: the same values up to rounding, and
+    # the state behind them in the slot; a second step goes on from it token by token
+    state[0].zero_()
+    o = torch.empty(T, nv, device="cuda")
+    sizes = [32, 32, 6]
+    chunks = [[0, sum(sizes[:c]), n, (1 if c == 0 else 0) | (2 if c == len(sizes) - 1 else 0)] for c, n in enumerate(sizes)]
+    ops.decay_scan(pj[:70], dc, state, dev([[0, 70, 0, 0]], torch.int32), o[:70], heads, dk, dv, cols, dev(chunks, torch.int32),
+                   dev([[0, 3]], torch.int32))
+    ops.decay_scan(pj[70:], dc, state, dev([[0, T - 70, 70, 0]], torch.int32), o[70:], heads, dk, dv, cols)
+    assert np.abs(f64(o).reshape(T, heads, dv) - want).max() < 2e-5 * scale
+    assert np.abs(f64(state[0]).reshape(heads, dk, dv) - S).max() < 2e-5 * np.abs(S).max()
     # two requests in one step, the second starting in the middle of the rows
     state[0].zero_()
     state[2].zero_()

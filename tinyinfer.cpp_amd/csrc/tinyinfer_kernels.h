@@ -231,6 +231,11 @@ int ti_gated_attention_rows(int dtype, const void* q, const void* pool, const in
 // [slots][heads][dk][dv]; entry_meta [n_entries][4] = (row0, tokens, start, slot); o f32 [M, heads dv]
 int ti_decay_scan(const float* proj, int ld, int off_q, int off_k, int off_v, const float* decay, float* state, long slot_stride,
                   const int* entry_meta, int n_entries, float* o, int heads, int dk, int dv, hipStream_t stream);
+// the same with the entries' tokens in chunks that run side by side (chunks [n_chunks][4] = (entry, first row, tokens, 1: the
+// entry's first chunk + 2: its last), spans [n_entries][2] = (first chunk, chunks); scratch float [n_chunks][heads][dk dv])
+int ti_decay_scan_chunked(const float* proj, int ld, int off_q, int off_k, int off_v, const float* decay, float* state,
+                          long slot_stride, const int* entry_meta, int n_entries, const int* chunks, int n_chunks, const int* spans,
+                          float* scratch, float* o, int heads, int dk, int dv, hipStream_t stream);
 // out = o / rms(o over the whole row) * w * sigmoid(gate), gate in rows of ld floats from column off_g on
 int ti_gated_row_norm(int out_dtype, const float* o, const float* gate, int ld, int off_g, const float* w, void* out, int M, int W,
                       float eps, hipStream_t stream);

@@ -1299,7 +1299,11 @@ int ti_ops_call(void* ops_, const char* op_, const ti_tensor* t, int n_t, const 
     c.q = (int)num(3);
     c.k = (int)num(4);
     c.v = (int)num(5);
-    ops.decay_scan(arg(0), c, arg(1), arg(2), iptr(3), (int)arg(3).shape[0], arg(4), (int)num(0), (int)num(1), (int)num(2));
+    // optional: chunks [n][4] and spans [R][2] (tensors 5 and 6): the chunked form
+    const bool chunked = n_t > 6 && arg(5).defined();
+    ops.decay_scan(arg(0), c, arg(1), arg(2), iptr(3), (int)arg(3).shape[0], arg(4), (int)num(0), (int)num(1), (int)num(2),
+                   chunked ? iptr(5) : nullptr, chunked ? (int)arg(5).shape[0] : 0, chunked ? iptr(6) : nullptr,
+                   chunked ? &workspace_of(&ops) : nullptr);
   } else if (op == "gated_row_norm") {
     // o, proj, w, out; gate column, eps
     ops.gated_row_norm(arg(0), arg(1), (int)num(0), arg(2), (float)num(1), arg(3));

@@ -424,8 +424,11 @@ class Ops {
                        float scale, int window, const AttentionWork* work = nullptr, Workspace* ws = nullptr);
   // Linear attention with a fixed decay per head over each entry's tokens, from and into its state slot: S <- decay_h S + k v^T,
   // o = S^T q with q, k, v = silu of proj's columns; decay f32 [heads]; state f32 [slots][heads][dk dv]; o f32 [M, heads dv]
+  // chunks (device int32 [n_chunks][4] = (entry, first row, tokens, 1: the entry's first chunk + 2: its last)) and spans
+  // ([n_entries][2] = (first chunk, chunks)): long portions run as chunks side by side, through scratch of `ws`
   void decay_scan(const Tensor& proj, const QkvColumns& cols, const Tensor& decay, const Tensor& state, const int* entry_meta,
-                  int n_entries, const Tensor& o, int heads, int dk, int dv);
+                  int n_entries, const Tensor& o, int heads, int dk, int dv, const int* chunks = nullptr, int n_chunks = 0,
+                  const int* spans = nullptr, Workspace* ws = nullptr);
   // out = o / rms(o over the whole row) * w * sigmoid(gate columns of proj), in the compute dtype
   void gated_row_norm(const Tensor& o, const Tensor& proj, int gate_col, const Tensor& w, float eps, const Tensor& out);
   // ---- layers that norm what a sublayer returns; short convolutions; differential attention; mixtures of experts

@@ -454,9 +454,11 @@ class Ops:
         self._call("gated_attention", [q, pool, table, positions, slots, sink, gate_proj, out],
                    [heads, kv_heads, dk, dv, scale, int(window or 0), gate_col, gate_mode])
 
-    def decay_scan(self, proj, decay, state, entries, o, heads, dk, dv, columns):
-        """entries int32 [R, 4] = (first row, tokens, -, state slot); S <- decay S + k v^T, o = S^T q on silu'd columns of proj."""
-        self._call("decay_scan", [proj, decay, state, entries, o], [heads, dk, dv] + list(columns))
+    def decay_scan(self, proj, decay, state, entries, o, heads, dk, dv, columns, chunks=None, spans=None):
+        """entries int32 [R, 4] = (first row, tokens, -, state slot); S <- decay S + k v^T, o = S^T q on silu'd columns of proj.
+        chunks int32 [n, 4] = (entry, first row, tokens, 1: the entry's first chunk + 2: its last) and spans int32 [R, 2] = (first
+        chunk, chunks): the entries' tokens run as chunks side by side."""
+        self._call("decay_scan", [proj, decay, state, entries, o, chunks, spans], [heads, dk, dv] + list(columns))
 
     def gated_row_norm(self, o, proj, gate_col, w, eps, out):
         self._call("gated_row_norm", [o, proj, w, out], [gate_col, eps])

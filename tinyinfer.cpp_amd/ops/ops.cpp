@@ -1314,8 +1314,9 @@ void Ops::gated_attention(const Tensor& q, const Tensor& pool, const CacheView& 
 }
 
 void Ops::decay_scan(const Tensor& proj, const QkvColumns& cols, const Tensor& decay, const Tensor& state, const int* entry_meta,
-                     int n_entries, const Tensor& o, int heads, int dk, int dv) {
-  TIMED("decay_scan " + dims(proj) + " entries=" + std::to_string(n_entries));
+                     int n_entries, const Tensor& o, int heads, int dk, int dv, const int* chunks, int n_chunks, const int* spans,
+                     Workspace* ws) {
+  TIMED("decay_scan " + dims(proj) + " entries=" + std::to_string(n_entries) + (chunks ? " chunks=" + std::to_string(n_chunks) : ""));
   require(proj.ndim == 2 && proj.dtype == DType::F32 && proj.contiguous(), "decay_scan: proj must be contiguous float32 [M, N]");
   const int64_t per_slot = (int64_t)heads * dk * dv;
   require(state.dtype == DType::F32 && state.contiguous() && state.ndim >= 2 && state.numel() == state.shape[0] * per_slot,
@@ -1324,6 +1325,17 @@ void Ops::decay_scan(const Tensor& proj, const QkvColumns& cols, const Tensor& d
   require(o.dtype == DType::F32 && o.contiguous() && o.ndim == 2 && o.shape[0] == proj.shape[0] && o.shape[1] == (int64_t)heads * dv,
           "decay_scan: o " + o.describe() + " does not fit");
   require(entry_meta != nullptr || n_entries == 0, "decay_scan: no entry records");
+  if (chunks) {
+    require(spans && ws && n_chunks >= n_entries, "decay_scan: chunks need spans and a workspace");
+    float* scratch = (float*)ws->get("decay.chunk_states", (size_t)n_chunks * per_slot * 4);
+    int rc = KERNEL("linear_attention", ti_decay_scan_chunked)((const float*)proj.data, (int)proj.shape[1], cols.q, cols.k, cols.v,
+                                                               (const float*)decay.data, (float*)state.data, (long)per_slot, entry_meta,
+                                                               n_entries, chunks, n_chunks, spans, scratch, (float*)o.data, heads, dk, dv,
+                                                               (hipStream_t)launch_stream());
+    check("linear_attention", rc, "decay_scan(chunked)");
+    took("[chunked]");
+    return;
+  }
   int rc = KERNEL("linear_attention", ti_decay_scan)((const float*)proj.data, (int)proj.shape[1], cols.q, cols.k, cols.v,
                                                      (const float*)decay.data, (float*)state.data, (long)per_slot, entry_meta, n_entries,
                                                      (float*)o.data, heads, dk, dv, (hipStream_t)launch_stream());

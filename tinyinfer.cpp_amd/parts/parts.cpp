@@ -2488,6 +2488,36 @@ class DecayAttention final : public MixerPart {
     n.state_shape = {heads, (int64_t)dk * dv};
     return n;
   }
+  // A step with a long portion: every entry's tokens in chunks of CHUNK that run side by side (the state is carried from chunk
+  // to chunk element by element), from CHUNK_FROM tokens on.  The lists are the same for every such mixer of the model; the
+  // first one builds them.
+  static constexpr int CHUNK = 64, CHUNK_FROM = 128;
+  void plan(StepPlan& plan) const override {
+    if (plan.decode_only() || plan.has("decay.chunks")) return;
+    const auto& entries = plan.entries();
+    int longest = 0;
+    size_t n_chunks = 0;
+    for (const auto& e : entries) {
+      longest = std::max(longest, e.n_tokens);
+      n_chunks += (size_t)(e.n_tokens + CHUNK - 1) / CHUNK;
+    }
+    if (longest < CHUNK_FROM) return;
+    int* chunks = plan.ints("decay.chunks", 4 * n_chunks);
+    int* spans = plan.ints("decay.spans", 2 * entries.size());
+    int c = 0;
+    for (size_t i = 0; i < entries.size(); ++i) {
+      const auto& e = entries[i];
+      const int n = (e.n_tokens + CHUNK - 1) / CHUNK;
+      spans[2 * i] = c;
+      spans[2 * i + 1] = n;
+      for (int k = 0; k < n; ++k, ++c) {
+        chunks[4 * c] = (int)i;
+        chunks[4 * c + 1] = e.row0 + k * CHUNK;
+        chunks[4 * c + 2] = std::min(CHUNK, e.n_tokens - k * CHUNK);
+        chunks[4 * c + 3] = (k == 0 ? 1 : 0) | (k == n - 1 ? 2 : 0);
+      }
+    }
+  }
   void run(StepContext& ctx, const Rows& h, const Tensor& out, Ops::Epilogue epi) {
     const int64_t M = h.t.shape[0];
     Tensor proj = ctx.buf("decay.proj", DType::F32, {M, width});
@@ -2499,7 +2529,8 @@ class DecayAttention final : public MixerPart {
     cols.q = 0;
     cols.k = (int)nq;
     cols.v = (int)(2 * nq);
-    ctx.ops.decay_scan(proj, cols, w_decay, state, ctx.entry_meta, (int)ctx.entries.size(), o, heads, dk, dv);
+    ctx.ops.decay_scan(proj, cols, w_decay, state, ctx.entry_meta, (int)ctx.entries.size(), o, heads, dk, dv, ctx.planned("decay.chunks"),
+                       (int)(ctx.planned_size("decay.chunks") / 4), ctx.planned("decay.spans"), &ctx.ws);
     Tensor a = ctx.buf("decay.gated", ctx.act_dtype, {M, nv});
     ctx.ops.gated_row_norm(o, proj, (int)(2 * nq + nv), norm_w, eps, a);
     ctx.ops.linear(a, w_o, out, epi, epi == Ops::Add);
