@@ -102,6 +102,22 @@ def test_streams_read_and_written(ops, S):
     ops.hyper_write(streams, dev(mix), dev(back), dev(y))
     want = np.einsum("st,smw->tmw", m32, x32) + b32[:, None, None] * y32[None]
     assert np.abs(f64(streams) - want).max() < 1e-5 * max(1.0, np.abs(want).max())
+    # two branches left apart and the next sublayer's read in the same pass: the same bits as the kernels one after the other
+    y2 = rng.normal(size=(M, W))
+    a, b = dev(xs), dev(xs)
+    both = torch.empty(M, W, device="cuda")
+    ops.scaled_add(both.zero_(), dev(y), torch.full((W,), 0.6, device="cuda"), dev(y2), torch.full((W,), 0.5, device="cuda"))
+    want2 = np.einsum("st,smw->tmw", m32, x32) + b32[:, None, None] * (0.6 * y32 + 0.5 * f32_round(y2))[None]
+    for dtype in ("float32", "bfloat16"):
+        a.copy_(dev(xs))
+        b.copy_(dev(xs))
+        out1 = torch.empty(M, W, device="cuda", dtype=DT[dtype])
+        out2 = torch.empty(M, W, device="cuda", dtype=DT[dtype])
+        ops.hyper_write(a, dev(mix), dev(back), dev(y), dev(y2), 0.6, 0.5)
+        ops.layernorm_mixed(a, dev(coef), dev(g), 1e-6, out1)
+        ops.hyper_write(b, dev(mix), dev(back), dev(y), dev(y2), 0.6, 0.5, dev(coef), dev(g), 1e-6, out2)
+        assert np.abs(f64(a) - want2).max() < 1e-5 * max(1.0, np.abs(want2).max())
+        assert np.array_equal(f64(a), f64(b)) and np.array_equal(f64(out1), f64(out2))
     x0 = dev(y)
     ops.hyper_spread(x0, streams)
     assert all(np.array_equal(f64(streams[s]), f64(x0)) for s in range(S))

@@ -204,9 +204,13 @@ int ti_mixed_layernorm(int out_dtype, const float* x, long stream_stride, int S,
 int ti_hyper_combine(const float* x, long stream_stride, int S, const float* coef, float* u, long n, hipStream_t stream);
 // every stream a copy of x
 int ti_hyper_spread(const float* x, float* streams, long stream_stride, int S, long n, hipStream_t stream);
-// x_t <- sum_s mix[s, t] x_s + back[t] y, every t at once from the old streams
-int ti_hyper_write(float* streams, long stream_stride, int S, const float* mix, const float* back, const float* y, long n,
-                   hipStream_t stream);
+// x_t <- sum_s mix[s, t] x_s + back[t] y, every t at once from the old streams; y2 (null: none): the output is f1 y + f2 y2
+int ti_hyper_write(float* streams, long stream_stride, int S, const float* mix, const float* back, const float* y, const float* y2,
+                   float f1, float f2, long n, hipStream_t stream);
+// the same write and, in the same pass, out = layernorm(sum_t coef[t] x_t) * w of the new streams (what ti_mixed_layernorm gives)
+int ti_hyper_write_read(int out_dtype, float* streams, long stream_stride, int S, const float* mix, const float* back, const float* y,
+                        const float* y2, float f1, float f2, const float* coef, const float* w, void* out, int M, int H, float eps,
+                        hipStream_t stream);
 
 // ---- libti_gated_attention: attention with per-head norms, values from the keys or mixed with another layer's, a sink, a gate
 // proj f32 [M, ld] holds q (n_head x dk), k (n_kv x dk) and v (n_kv x dv; off_v < 0: the values are the keys as projected) from

@@ -1267,7 +1267,9 @@ int ti_ops_call(void* ops_, const char* op_, const ti_tensor* t, int n_t, const 
   } else if (op == "hyper_spread") {
     ops.hyper_spread(arg(0), arg(1));               // x, streams
   } else if (op == "hyper_write") {
-    ops.hyper_write(arg(0), arg(1), arg(2), arg(3));      // streams, mix, back, y
+    // streams, mix, back, y, [y2, next coef, next weight, next rows]; [f1, f2, eps]
+    ops.hyper_write(arg(0), arg(1), arg(2), arg(3), n_t > 4 ? arg(4) : Tensor(), n_s > 0 ? (float)num(0) : 1.f, n_s > 1 ? (float)num(1) : 1.f,
+                    n_t > 5 ? arg(5) : Tensor(), n_t > 6 ? arg(6) : Tensor(), n_s > 2 ? (float)num(2) : 0.f, n_t > 7 ? arg(7) : Tensor());
   } else if (op == "gated_qkv_prep") {
     // proj, q_w, k_w, inv_freq, rope_table, positions, slots, table, pool, q_out, lambda, kept; eps, heads, kv_heads, dk, dv,
     // columns of q, k, v (v < 0: the values are the keys), rotated entries, mix mode

@@ -404,7 +404,12 @@ class Ops {
   void hyper_combine(const Tensor& streams, const Tensor& coef, const Tensor& u);
   void hyper_spread(const Tensor& x, const Tensor& streams);                       // every stream a copy of x
   // streams[t] <- sum_s mix[s, t] streams[s] + back[t] y, every t at once from the old streams (mix f32 [S, S], back f32 [S])
-  void hyper_write(const Tensor& streams, const Tensor& mix, const Tensor& back, const Tensor& y);
+  // y2 (undefined: none): the sublayer's output is f1 y + f2 y2, two branches left apart.  next_coef, next_w, next_out (all three
+  // or none): in the same pass next_out = layernorm(sum_t next_coef[t] streams[t]) * next_w of the new streams (what
+  // layernorm_mixed gives: same arithmetic, same order)
+  void hyper_write(const Tensor& streams, const Tensor& mix, const Tensor& back, const Tensor& y, const Tensor& y2 = Tensor(),
+                   float f1 = 1.f, float f2 = 1.f, const Tensor& next_coef = Tensor(), const Tensor& next_w = Tensor(), float eps = 0.f,
+                   const Tensor& next_out = Tensor());
   // What a gated attention layer does to the 32-bit sums of its stacked projection before the attention itself: proj f32 [M, N]
   // holds q (heads x dk), k (kv_heads x dk) and v (kv_heads x dv) from the given columns on (off_v < 0: the values are the keys as
   // projected, before norm and rotation).  q_w / k_w (undefined: none): an RMS norm of every head with a weight of dk shared by the
@@ -714,7 +719,9 @@ class NormPart : public Part { public: using Part::Part; const char* family() co
   // the norm of u = sum_s coef[s] streams[s] (streams f32 [S, M, dim], coef f32 [S]) without u being formed: for arrangements
   // that keep the residual in several streams
   virtual bool can_mix() const { return false; }
-  virtual Rows forward_mixed(StepContext& ctx, const Tensor& streams, const Tensor& coef); };
+  virtual Rows forward_mixed(StepContext& ctx, const Tensor& streams, const Tensor& coef);
+  // for a writer of the streams that takes the next read in: the norm's weight, eps and the rows it would write (null: no such form)
+  virtual bool mixed_form(StepContext& ctx, int64_t M, Tensor& weight, float& eps, Rows& rows) { return false; } };
 class PositionPart : public Part { public: using Part::Part; const char* family() const override { return "pos"; }
   virtual bool fused(Ops::Rotation& rot) const { return false; }    // arguments for the fused q/k kernels
   virtual bool additive() const { return false; }                   // an encoding added to the residual behind the embedding ...
@@ -725,7 +732,11 @@ class MixerPart : public Part { public: using Part::Part; const char* family() c
   // y f32 [M, H] = the part's output, nothing added: for arrangements that scale or combine outputs before the sum
   virtual bool can_store() const { return false; }
   virtual void forward_store(StepContext& ctx, const Rows& h, const Tensor& y);
-  virtual bool takes_lazy_norm() const { return false; } };        // h goes into exactly one Ops::linear
+  virtual bool takes_lazy_norm() const { return false; }         // h goes into exactly one Ops::linear
+  // a mixer whose output is f1 y1 + f2 y2 may leave the two apart for a reader that adds them on its way (an arrangement that
+  // scales or mixes outputs anyway): y1, y2 f32 [M, H]
+  virtual bool leaves_pair() const { return false; }
+  virtual void forward_pair(StepContext& ctx, const Rows& h, const Tensor& y1, const Tensor& y2, float& f1, float& f2); };
 // an operation along time on every channel of the step's rows, with what it must remember of a request as its state
 class FilterPart : public Part { public: using Part::Part; const char* family() const override { return "filter"; }
   virtual void forward(StepContext& ctx, const Tensor& u, const Tensor& out) = 0;

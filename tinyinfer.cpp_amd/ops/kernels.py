@@ -436,9 +436,10 @@ class Ops:
     def hyper_spread(self, x, streams):
         self._call("hyper_spread", [x, streams])
 
-    def hyper_write(self, streams, mix, back, y):
-        """streams[t] <- sum_s mix[s, t] streams[s] + back[t] y, every t at once."""
-        self._call("hyper_write", [streams, mix, back, y])
+    def hyper_write(self, streams, mix, back, y, y2=None, f1=1.0, f2=1.0, next_coef=None, next_w=None, eps=0.0, next_out=None):
+        """streams[t] <- sum_s mix[s, t] streams[s] + back[t] y, every t at once; with y2 the output is f1 y + f2 y2; with next_*
+        the same pass leaves next_out = layernorm(sum_t next_coef[t] streams[t]) * next_w of the new streams."""
+        self._call("hyper_write", [streams, mix, back, y, y2, next_coef, next_w, next_out], [f1, f2, eps])
 
     def gated_qkv_prep(self, proj, q_w, k_w, inv_freq, rope_table, positions, slots, table, pool, q_out, heads, kv_heads, dk, dv, columns,
                        eps=1e-6, rot_dims=0, mix_mode=0, mix_lambda=None, kept=None):

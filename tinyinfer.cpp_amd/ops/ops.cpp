@@ -1238,15 +1238,28 @@ void Ops::hyper_spread(const Tensor& x, const Tensor& streams) {
   check("hyper", rc, "hyper_spread");
 }
 
-void Ops::hyper_write(const Tensor& streams, const Tensor& mix, const Tensor& back, const Tensor& y) {
-  TIMED("hyper_write " + dims(streams));
+void Ops::hyper_write(const Tensor& streams, const Tensor& mix, const Tensor& back, const Tensor& y, const Tensor& y2, float f1, float f2,
+                      const Tensor& next_coef, const Tensor& next_w, float eps, const Tensor& next_out) {
+  TIMED("hyper_write " + dims(streams) + (y2.defined() ? " pair" : "") + (next_out.defined() ? " +read" : ""));
   check_streams("hyper_write", streams);
-  const int64_t S = streams.shape[0], n = streams.shape[1] * streams.shape[2];
+  const int64_t S = streams.shape[0], M = streams.shape[1], H = streams.shape[2], n = M * H;
   require(mix.dtype == DType::F32 && mix.numel() == S * S && mix.contiguous() && back.dtype == DType::F32 && back.numel() == S &&
-              y.dtype == DType::F32 && y.contiguous() && y.numel() == n,
+              y.dtype == DType::F32 && y.contiguous() && y.numel() == n && (!y2.defined() || (y2.dtype == DType::F32 && y2.contiguous() && y2.numel() == n)),
           "hyper_write: mix " + mix.describe() + ", back " + back.describe() + " or y " + y.describe() + " do not fit");
+  const float* second = y2.defined() ? (const float*)y2.data : nullptr;
+  if (next_out.defined()) {
+    require(next_coef.dtype == DType::F32 && next_coef.numel() == S && next_w.dtype == DType::F32 && next_w.numel() == H &&
+                next_out.ndim == 2 && next_out.shape[0] == M && next_out.shape[1] == H && next_out.contiguous(),
+            "hyper_write: the next read's coefficients, weight or rows do not fit");
+    int rc = KERNEL("hyper", ti_hyper_write_read)(code(next_out.dtype, "hyper_write"), (float*)streams.data, (long)n, (int)S,
+                                                  (const float*)mix.data, (const float*)back.data, (const float*)y.data, second, f1, f2,
+                                                  (const float*)next_coef.data, (const float*)next_w.data, next_out.data, (int)M, (int)H,
+                                                  eps, (hipStream_t)launch_stream());
+    check("hyper", rc, "hyper_write(+read)");
+    return;
+  }
   int rc = KERNEL("hyper", ti_hyper_write)((float*)streams.data, (long)n, (int)S, (const float*)mix.data, (const float*)back.data,
-                                           (const float*)y.data, (long)n, (hipStream_t)launch_stream());
+                                           (const float*)y.data, second, f1, f2, (long)n, (hipStream_t)launch_stream());
   check("hyper", rc, "hyper_write");
 }
 

@@ -128,6 +128,9 @@ void NormPart::forward_add(StepContext&, const Tensor&, const Tensor&, bool, con
 Rows NormPart::forward_mixed(StepContext&, const Tensor&, const Tensor&) {
   throw EngineError(std::string("the norm '") + kind_name() + "' has no form for a sum of streams");
 }
+void MixerPart::forward_pair(StepContext&, const Rows&, const Tensor&, const Tensor&, float&, float&) {
+  throw EngineError(std::string("the mixer '") + kind_name() + "' does not leave its output as a pair");
+}
 void MixerPart::forward_store(StepContext&, const Rows&, const Tensor&) {
   throw EngineError(std::string("the mixer '") + kind_name() + "' cannot write its output apart from the residual");
 }
@@ -2298,6 +2301,13 @@ class LayerNorm final : public NormPart {
     ctx.ops.layernorm_mixed(streams, coef, weight, eps, r.t);
     return r;
   }
+  bool mixed_form(StepContext& ctx, int64_t M, Tensor& w, float& e, Rows& rows) override {
+    w = weight;
+    e = eps;
+    rows = Rows();
+    rows.t = ctx.buf("norm.out", ctx.act_dtype, {M, dim});
+    return true;
+  }
   std::vector<std::pair<std::string, Tensor>> held() const override { return {{"weight", weight}}; }
   int64_t dim = 0;
   float eps = 1e-6f;
@@ -2409,11 +2419,30 @@ class HyperBlock final : public BlockPart {
   void forward(StepContext& ctx, const Tensor& x) override {
     const int64_t M = x.shape[0];
     const Tensor xs = hyper_streams(ctx, streams, M, dim);
-    Tensor y = ctx.buf("hyper.y", DType::F32, {M, dim});
-    mixer->forward_store(ctx, read(ctx, *norm1, xs, w_in[0]), y);
-    ctx.ops.hyper_write(xs, w_mix[0], w_out[0], y);
-    if (!ffn) return;
-    ffn->forward_store(ctx, read(ctx, *norm2, xs, w_in[1]), y);
+    Tensor y = ctx.buf("hyper.y", DType::F32, {M, dim}), y2;
+    const Rows h = read(ctx, *norm1, xs, w_in[0]);
+    float f1 = 1.f, f2 = 1.f;
+    if (mixer->leaves_pair()) {      // two branches left apart: the write adds them on its way
+      y2 = ctx.buf("hyper.y2", DType::F32, {M, dim});
+      mixer->forward_pair(ctx, h, y, y2, f1, f2);
+    } else {
+      mixer->forward_store(ctx, h, y);
+    }
+    if (!ffn) {
+      ctx.ops.hyper_write(xs, w_mix[0], w_out[0], y, y2, f1, f2);
+      return;
+    }
+    // the mixer's write and the feed-forward's read in one pass over the streams, where the norm has a form for that
+    Tensor nw;
+    float neps = 0.f;
+    Rows h2;
+    if (norm2->mixed_form(ctx, M, nw, neps, h2)) {
+      ctx.ops.hyper_write(xs, w_mix[0], w_out[0], y, y2, f1, f2, w_in[1], nw, neps, h2.t);
+    } else {
+      ctx.ops.hyper_write(xs, w_mix[0], w_out[0], y, y2, f1, f2);
+      h2 = read(ctx, *norm2, xs, w_in[1]);
+    }
+    ffn->forward_store(ctx, h2, y);
     ctx.ops.hyper_write(xs, w_mix[1], w_out[1], y);
   }
   std::vector<std::pair<std::string, Tensor>> held() const override {
@@ -2591,6 +2620,13 @@ class SumMixer final : public MixerPart {
   void forward_store(StepContext& ctx, const Rows& h, const Tensor& y) override {
     ctx.ops.fill_zero(y.data, y.bytes());
     run(ctx, h, y);
+  }
+  bool leaves_pair() const override { return true; }
+  void forward_pair(StepContext& ctx, const Rows& h, const Tensor& y1, const Tensor& y2, float& f1, float& f2) override {
+    left->forward_store(ctx, h, y1);
+    right->forward_store(ctx, h, y2);
+    f1 = left_scale;
+    f2 = right_scale;
   }
   std::shared_ptr<MixerPart> left, right;
   int64_t dim = 0;
