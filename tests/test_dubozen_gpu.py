@@ -449,7 +449,7 @@ def make_trace(mode, requests):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name,page_size", [("streams", 8), ("plain", 4), ("wide", 16), ("single", 16)])
+@pytest.mark.parametrize("name,page_size", [("streams", 8), ("plain", 4), ("wide", 16), ("single", 16), ("squares", 16)])
 @pytest.mark.parametrize("mode", ["whole", "tail", "portions", "mixed"])
 def test_engine_matches_plain(folders, name, page_size, dtype, mode):
     folder, requests, want, _ = folders(name)

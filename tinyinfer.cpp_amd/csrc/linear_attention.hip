@@ -14,7 +14,8 @@
 
 TI_ERROR_API
 
-__device__ __forceinline__ float la_silu(float z) { return z / (1.0f + expf(-z)); }
+// z sigmoid(z) with the hardware's exponential and reciprocal (a few units of 32-bit rounding)
+__device__ __forceinline__ float la_silu(float z) { return z * __frcp_rn(1.0f + __expf(-z)); }
 
 // MODE 0: an entry's tokens from and into its slot.  MODE 1: a chunk alone from an empty state, no outputs, its state into
 // `scratch` [chunk][head][dk][dv].  MODE 2: a chunk from the state `scratch` holds for it (what the carry kernel left there),
@@ -125,13 +126,29 @@ __global__ void decay_carry_kernel(float* __restrict__ scratch, const int* __res
   float* slot = state + (size_t)entry_meta[4 * e + 3] * slot_stride + (size_t)h * per_head + x;
   const float a = decay[h];
   float S = *slot;
-  for (int c = c0; c < c0 + nc; ++c) {
-    float* at = scratch + ((size_t)c * heads + h) * per_head + x;
-    const float add = *at;
-    *at = S;
-    float f = 1.f;
-    for (int t = chunks[4 * c + 2]; t > 0; --t) f *= a;
-    S = fmaf(f, S, add);
+  int f_len = -1;      // the power of the decay last worked out, and for how many tokens
+  float f = 1.f;
+  // eight chunks' shares are asked for together: the walk waits for memory once per eight chunks, not once per chunk
+  for (int c = c0; c < c0 + nc; c += 8) {
+    float add[8];
+    int len[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int ci = min(c + i, c0 + nc - 1);
+      add[i] = scratch[((size_t)ci * heads + h) * per_head + x];
+      len[i] = chunks[4 * ci + 2];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (c + i >= c0 + nc) break;
+      scratch[((size_t)(c + i) * heads + h) * per_head + x] = S;
+      if (len[i] != f_len) {
+        f = 1.f;
+        for (int t = len[i]; t > 0; --t) f *= a;
+        f_len = len[i];
+      }
+      S = fmaf(f, S, add[i]);
+    }
   }
   *slot = S;
 }
