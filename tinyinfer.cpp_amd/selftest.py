@@ -464,6 +464,79 @@ def case_diff_attention(ops, rng, nh, nkv, dk, dv, T, block, taps, rot, dtype, P
     return fails
 
 
+def case_streams_gates_and_decay(ops, rng) -> int:
+    """The layer norm of a weighted sum of streams, the write into the streams, attention with a sink and a gate over pages,
+    and linear attention with a fixed decay whole and in chunks, each against a host computation."""
+    fails = 0
+
+    def D(a):      # 64-bit host arrays go to the device as float32, integer lists as they are
+        a = np.asarray(a)
+        return _dev(a.astype(np.float32) if a.dtype == np.float64 else a)
+
+    S, M, W = 3, 21, 70
+    xs, coef, back = rng.normal(size=(S, M, W)), rng.normal(0.5, 0.4, size=S), rng.normal(1.0, 0.4, size=S)
+    mix, g, y = np.eye(S) + rng.normal(0, 0.3, size=(S, S)), rng.normal(1.0, 0.2, size=W), rng.normal(size=(M, W))
+    f32 = lambda a: np.asarray(a, dtype=np.float32).astype(np.float64)
+    u = np.einsum("s,smw->mw", f32(coef), f32(xs))
+    d = u - u.mean(-1, keepdims=True)
+    want = d / np.sqrt((d * d).mean(-1, keepdims=True) + 1e-6) * f32(g)
+    streams, out = D(xs), torch.empty(M, W, device="cuda")
+    ops.layernorm_mixed(streams, D(coef), D(g), 1e-6, out)
+    fails += _say("layer norm of a weighted sum of 3 streams", float(np.abs(_f64(out) - want).max()), 5e-5)
+    ops.hyper_write(streams, D(mix), D(back), D(y))
+    want = np.einsum("st,smw->tmw", f32(mix), f32(xs)) + f32(back)[:, None, None] * f32(y)[None]
+    fails += _say("write into 3 streams", float(np.abs(_f64(streams) - want).max()), 2e-5)
+    # attention with a sink and a gate a head, keys 24 and values 40, pages of 8
+    T, nh, nkv, dk, dv, P = 70, 4, 2, 24, 40, 8
+    nq, nk, nv = nh * dk, nkv * dk, nkv * dv
+    proj = rng.normal(size=(T, nq + nk + nv + nh))
+    sink = rng.normal(0.5, 1.0, size=nh)
+    n_pages = -(-T // P)
+    table = rng.permutation(n_pages + 2)[:n_pages].astype(np.int32)[None, :]
+    pos, slots = np.arange(T, dtype=np.int32), np.zeros(T, dtype=np.int32)
+    for dtype, tol in ((torch.float32, 5e-5), (torch.bfloat16, 3e-2)):
+        pool = torch.zeros(n_pages + 2, nkv, P, dk + dv, device="cuda", dtype=dtype)
+        q_out = torch.empty(T, nq, device="cuda", dtype=dtype)
+        args = (D(pos), D(slots), D(table))
+        ops.gated_qkv_prep(D(proj), None, None, None, None, *args, pool, q_out, nh, nkv, dk, dv, (0, nq, nq + nk))
+        p32 = f32(proj)
+        rnd = _bf16 if dtype == torch.bfloat16 else (lambda a: a)
+        q, k = rnd(p32[:, :nq]).reshape(T, nh, dk), rnd(p32[:, nq:nq + nk]).reshape(T, nkv, dk)
+        v = rnd(p32[:, nq + nk:nq + nk + nv]).reshape(T, nkv, dv)
+        want = np.zeros((T, nh, dv))
+        for h in range(nh):
+            sc = q[:, h] @ k[:, h // 2].T * 0.2
+            sc[np.triu_indices(T, 1)] = -np.inf
+            m = np.maximum(sc.max(-1, keepdims=True), f32(sink)[h])
+            e = np.exp(sc - m)
+            want[:, h] = (e / (e.sum(-1, keepdims=True) + np.exp(f32(sink)[h] - m))) @ v[:, h // 2]
+            want[:, h] *= 1.0 / (1.0 + np.exp(-p32[:, nq + nk + nv + h]))[:, None]
+        out = torch.empty(T, nh * dv, device="cuda", dtype=dtype)
+        ops.gated_attention(q_out, pool, D(table), D(pos), D(slots), D(sink), D(proj), out, nh, nkv, dk, dv, 0.2,
+                            gate_col=nq + nk + nv, gate_mode=2)
+        fails += _say(f"attention with a sink and a gate, {str(dtype).split('.')[-1]}", float(np.abs(_f64(out).reshape(T, nh, dv) - want).max()), tol)
+    # linear attention with a decay: 150 tokens whole and in chunks of 64
+    heads, dk, dv, T = 2, 32, 48, 150
+    nq, nv = heads * dk, heads * dv
+    proj, decay = rng.normal(size=(T, 2 * nq + nv)) * 0.8, np.array([0.97, 0.6])
+    silu = lambda z: z / (1.0 + np.exp(-z))
+    p32 = f32(proj)
+    q, k, v = silu(p32[:, :nq]).reshape(T, heads, dk), silu(p32[:, nq:2 * nq]).reshape(T, heads, dk), silu(p32[:, 2 * nq:]).reshape(T, heads, dv)
+    want, St = np.zeros((T, heads, dv)), np.zeros((heads, dk, dv))
+    for t in range(T):
+        for h in range(heads):
+            St[h] = f32(decay)[h] * St[h] + np.outer(k[t, h], v[t, h])
+            want[t, h] = St[h].T @ q[t, h]
+    entries = D(np.array([[0, T, 0, 0]], dtype=np.int32))
+    for name, extra in (("whole", ()), ("in chunks", (D(np.array([[0, 0, 64, 1], [0, 64, 64, 0], [0, 128, 22, 2]], dtype=np.int32)),
+                                                     D(np.array([[0, 3]], dtype=np.int32))))):
+        state, o = torch.zeros(1, heads, dk * dv, device="cuda"), torch.empty(T, nv, device="cuda")
+        ops.decay_scan(D(proj), D(decay), state, entries, o, heads, dk, dv, (0, nq, 2 * nq), *extra)
+        fails += _say(f"linear attention with a decay, {name}", float(np.abs(_f64(o).reshape(T, heads, dv) - want).max()), 2e-5 * float(np.abs(want).max()))
+        fails += _say(f"  its state, {name}", float(np.abs(_f64(state).reshape(heads, dk, dv) - St).max()), 2e-5 * float(np.abs(St).max()))
+    return fails
+
+
 def run_selftest() -> int:
     if not torch.cuda.is_available():
         print("[selftest] no GPU: the kernels of this framework run on an AMD GPU (gfx950) only", flush=True)
@@ -491,6 +564,7 @@ def run_selftest() -> int:
     fails += case_diff_attention(ops, rng, nh=3, nkv=1, dk=20, dv=12, T=90, block=37, taps=3, rot=8, dtype=torch.float32, P=8)
     fails += case_diff_attention(ops, rng, nh=4, nkv=2, dk=32, dv=64, T=200, block=150, taps=4, rot=32, dtype=torch.bfloat16)
     fails += case_diff_attention(ops, rng, nh=8, nkv=1, dk=64, dv=128, T=130, block=64, taps=2, rot=16, dtype=torch.bfloat16)
+    fails += case_streams_gates_and_decay(ops, rng)
     fails += case_embed_argmax_sample(ops, rng)
     fails += case_model_shapes(ops, rng)
     fails += case_head_bandwidth(ops, rng)
