@@ -152,12 +152,16 @@ Json dubozen_typed_config(const Json& d) {
       rm.set("dim", dim);
       rm.set("vdim", vdim);
       const Json& decay = need(right, "decay", rw);
-      if (decay.type() != Json::Array || (int64_t)decay.size() != heads)
-        throw ConfigError("config.json: " + rw + "'decay' must list one number a head (" + std::to_string(heads) + ")");
       Json dl = Json::array();
-      for (const Json& v : decay.items()) {
-        if (!v.is_number()) throw ConfigError("config.json: " + rw + "'decay' must hold numbers, got " + v.dump());
-        dl.push(Json(v.as_double()));
+      if (decay.is_number()) {      // one number: every head's
+        for (int64_t j = 0; j < heads; ++j) dl.push(Json(decay.as_double()));
+      } else {
+        if (decay.type() != Json::Array || (int64_t)decay.size() != heads)
+          throw ConfigError("config.json: " + rw + "'decay' must list one number a head (" + std::to_string(heads) + ")");
+        for (const Json& v : decay.items()) {
+          if (!v.is_number()) throw ConfigError("config.json: " + rw + "'decay' must hold numbers, got " + v.dump());
+          dl.push(Json(v.as_double()));
+        }
       }
       rm.set("decay", dl);
       mo.set("right", rm);
@@ -264,6 +268,7 @@ ModelSpec dubozen_spec(const Json& config) {
     if (S) {
       ls.block.params.set("streams", S);
       ls.block.params.set("dim", H);
+      ls.block.params.set("defer_write", true);      // the block that sums the streams closes the run of layers
     }
     ls.parts.emplace_back("norm1", norm(ls.prefix + ".norm1"));
     const std::string at = ls.prefix + ".mix";

@@ -659,6 +659,12 @@ class StepContext {
   size_t planned_size(const std::string& key) const;
   int64_t value(const std::string& key, int64_t fallback = 0) const;
 
+  // What a part leaves for a later part of the same step: a piece of work it has not done, for a part that can take it into a
+  // kernel of its own (a write into the streams of a residual, taken in by the next read of them).  Whoever finds a note does the
+  // work or takes it in, and removes the note.
+  struct Note { std::vector<Tensor> tensors; std::vector<double> numbers; };
+  std::map<std::string, Note> notes;
+
   Engine* engine = nullptr;               // null for a part run on its own
   const StepPlan* plan = nullptr;
   const int* meta_dev = nullptr;

@@ -2321,12 +2321,29 @@ class LayerNorm final : public NormPart {
 static Tensor hyper_streams(StepContext& ctx, int64_t streams, int64_t M, int64_t dim) {
   return ctx.buf("hyper.streams", DType::F32, {streams, M, dim});
 }
+// A layer may leave its last write into the streams as a note (`defer_write`): tensors (mix, back, y, y2 or undefined), numbers
+// (f1, f2).  The next layer's first read takes it in (one pass over the streams instead of two); whoever else needs the streams
+// complete does the write first.
+static const char* const HYPER_PENDING = "hyper.pending";
+static bool hyper_take_pending(StepContext& ctx, StepContext::Note& note) {
+  auto it = ctx.notes.find(HYPER_PENDING);
+  if (it == ctx.notes.end()) return false;
+  note = std::move(it->second);
+  ctx.notes.erase(it);
+  return true;
+}
+static void hyper_flush(StepContext& ctx, const Tensor& xs) {
+  StepContext::Note n;
+  if (hyper_take_pending(ctx, n))
+    ctx.ops.hyper_write(xs, n.tensors[0], n.tensors[1], n.tensors[2], n.tensors[3], (float)n.numbers[0], (float)n.numbers[1]);
+}
 class HyperSpreadBlock final : public BlockPart {
  public:
   HyperSpreadBlock(const std::string& prefix, const Json& p) : BlockPart(prefix), streams(param_int(p, "streams")), dim(param_int(p, "dim")) {}
   const char* kind_name() const override { return "hyper_spread"; }
   void forward(StepContext& ctx, const Tensor& x) override {
     ctx.ops.flush();
+    ctx.notes.erase(HYPER_PENDING);
     ctx.ops.hyper_spread(x, hyper_streams(ctx, streams, x.shape[0], dim));
   }
   int64_t streams, dim;
@@ -2337,7 +2354,9 @@ class HyperSumBlock final : public BlockPart {
   const char* kind_name() const override { return "hyper_sum"; }
   void forward(StepContext& ctx, const Tensor& x) override {
     ctx.ops.flush();
-    ctx.ops.hyper_combine(hyper_streams(ctx, streams, x.shape[0], dim), Tensor(), x);
+    const Tensor xs = hyper_streams(ctx, streams, x.shape[0], dim);
+    hyper_flush(ctx, xs);
+    ctx.ops.hyper_combine(xs, Tensor(), x);
   }
   int64_t streams, dim;
 };
@@ -2346,7 +2365,8 @@ class HyperSumBlock final : public BlockPart {
 // reads u = sum_s in_q[s] x_s through its norm, and its output y goes back into all streams at once:
 // x_t <- sum_s mix_q[s, t] x_s + out_q[t] y (mix indexed [from, to]).  Tensors: prefix + ".hc<q>.in" [S], ".hc<q>.out" [S],
 // ".hc<q>.mix" [S, S], held in 32-bit.  A norm that can take the weighted sum in does (no u is written); the sublayers write
-// apart from the residual.
+// apart from the residual.  The mixer's write takes the feed-forward's read in; with `defer_write` the layer's last write is left
+// as a note for the next layer's first read (or for `hyper_sum`), which takes it in the same way.
 class HyperBlock final : public BlockPart {
  public:
   HyperBlock(const std::string& prefix, const Json& p, const PartChildren& c) : BlockPart(prefix) {
@@ -2362,6 +2382,7 @@ class HyperBlock final : public BlockPart {
       throw ConfigError("block 'hyper': its mixer and feed-forward must be able to write their output apart from the residual");
     streams = param_int(p, "streams");
     dim = param_int(p, "dim");
+    defer_write = p.has("defer_write") && p.at("defer_write").as_bool();
     if (streams < 1 || streams > 16) throw ConfigError("block 'hyper': " + std::to_string(streams) + " streams are not served (1 to 16)");
   }
   const char* kind_name() const override { return "hyper"; }
@@ -2420,7 +2441,23 @@ class HyperBlock final : public BlockPart {
     const int64_t M = x.shape[0];
     const Tensor xs = hyper_streams(ctx, streams, M, dim);
     Tensor y = ctx.buf("hyper.y", DType::F32, {M, dim}), y2;
-    const Rows h = read(ctx, *norm1, xs, w_in[0]);
+    // the write the layer before left undone goes into this layer's first read, where the norm has a form for that
+    Rows h;
+    StepContext::Note left;
+    Tensor w1;
+    float eps1 = 0.f;
+    if (hyper_take_pending(ctx, left)) {
+      if (norm1->mixed_form(ctx, M, w1, eps1, h)) {
+        ctx.ops.hyper_write(xs, left.tensors[0], left.tensors[1], left.tensors[2], left.tensors[3], (float)left.numbers[0],
+                            (float)left.numbers[1], w_in[0], w1, eps1, h.t);
+      } else {
+        ctx.ops.hyper_write(xs, left.tensors[0], left.tensors[1], left.tensors[2], left.tensors[3], (float)left.numbers[0],
+                            (float)left.numbers[1]);
+        h = read(ctx, *norm1, xs, w_in[0]);
+      }
+    } else {
+      h = read(ctx, *norm1, xs, w_in[0]);
+    }
     float f1 = 1.f, f2 = 1.f;
     if (mixer->leaves_pair()) {      // two branches left apart: the write adds them on its way
       y2 = ctx.buf("hyper.y2", DType::F32, {M, dim});
@@ -2429,7 +2466,8 @@ class HyperBlock final : public BlockPart {
       mixer->forward_store(ctx, h, y);
     }
     if (!ffn) {
-      ctx.ops.hyper_write(xs, w_mix[0], w_out[0], y, y2, f1, f2);
+      if (defer_write) ctx.notes[HYPER_PENDING] = StepContext::Note{{w_mix[0], w_out[0], y, y2}, {f1, f2}};
+      else ctx.ops.hyper_write(xs, w_mix[0], w_out[0], y, y2, f1, f2);
       return;
     }
     // the mixer's write and the feed-forward's read in one pass over the streams, where the norm has a form for that
@@ -2443,7 +2481,8 @@ class HyperBlock final : public BlockPart {
       h2 = read(ctx, *norm2, xs, w_in[1]);
     }
     ffn->forward_store(ctx, h2, y);
-    ctx.ops.hyper_write(xs, w_mix[1], w_out[1], y);
+    if (defer_write) ctx.notes[HYPER_PENDING] = StepContext::Note{{w_mix[1], w_out[1], y, Tensor()}, {1.0, 1.0}};
+    else ctx.ops.hyper_write(xs, w_mix[1], w_out[1], y);
   }
   std::vector<std::pair<std::string, Tensor>> held() const override {
     return {{"in1", w_in[0]}, {"out1", w_out[0]}, {"mix1", w_mix[0]}, {"in2", w_in[1]}, {"out2", w_out[1]}, {"mix2", w_mix[1]}};
@@ -2452,6 +2491,7 @@ class HyperBlock final : public BlockPart {
   std::shared_ptr<MixerPart> mixer;
   std::shared_ptr<FeedForwardPart> ffn;
   int64_t streams = 1, dim = 0;
+  bool defer_write = false;     // `defer_write`: the layer's last write is left to the next reader of the streams (a `hyper` layer or `hyper_sum`)
   Tensor w_in[2], w_out[2], w_mix[2];
 };
 
