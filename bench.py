@@ -121,7 +121,7 @@ def nazorax_config(base, mixers, ffn, experts, top, window):
                 layers=[kinds[i % len(kinds)] for i in range(L)])
 
 
-def dubozen_config(base, mixers, ffn, experts, top, streams):
+def dubozen_config(base, mixers, ffn, experts, top, streams, value_size=0):
     """A Dubozen config.json with the layer widths of the Qwen3 configuration `base`."""
     H, F, hd = base["hidden_size"], base["intermediate_size"], base["head_dim"]
     heads, kv = base["num_attention_heads"], base["num_key_value_heads"]
@@ -130,7 +130,7 @@ def dubozen_config(base, mixers, ffn, experts, top, streams):
     mlp = dict(kind="dense", ff=F) if ffn == "dense" else dict(kind="moe", expert=dict(ff=ff), router=dict(
         experts=experts, top=top, scale=2.5, groups=dict(count=groups, keep=max(1, groups // 2))))
     softmax = dict(heads=heads, kv_heads=kv, dim=hd, vdim=hd, scale=hd ** -0.5, rot=dict(base=1000000.0, dims=hd // 2))
-    attention = dict(type="attention", mixer=dict(softmax, v_mix=True), mlp=mlp)
+    attention = dict(type="attention", mixer=dict(softmax, vdim=value_size or hd, v_mix=True), mlp=mlp)
     decay = [1.0 - 2.0 ** (-5.0 - 3.0 * j / max(1, kv - 1)) for j in range(kv)]
     parallel = dict(type="parallel", mixer=dict(left=softmax, right=dict(heads=kv, dim=hd, vdim=hd, decay=decay), left_scale=0.5, right_scale=0.5),
                     mlp=mlp)
@@ -462,6 +462,7 @@ def main() -> int:
     ap.add_argument("--experts", type=int, default=8, help="--design mumasun / nazorax / dubozen: experts per layer")
     ap.add_argument("--top", type=int, default=2, help="--design mumasun / nazorax / dubozen: experts a token takes")
     ap.add_argument("--ffn", choices=["dense", "moe"], default="moe", help="--design nazorax / dubozen: the feed-forward of its layers")
+    ap.add_argument("--value-size", type=int, default=0, help="--design dubozen: the value size of its attention layers (0: the head size)")
     ap.add_argument("--streams", type=int, default=2, help="--design dubozen: copies of the residual (0: one plain residual)")
     ap.add_argument("--window", type=int, default=1024, help="--design nazorax: positions an attention layer's window keeps")
     ap.add_argument("--mask-size", type=int, default=4096, help="--design mumasun: positions of a block of visible keys")
@@ -515,7 +516,7 @@ def main() -> int:
     if args.design == "dubozen":
         if args.mixers in ("mlstm", "latent"):
             ap.error("--design dubozen has the mixers attention, parallel and alternate")
-        cfg = dubozen_config(cfg, args.mixers, args.ffn, args.experts, args.top, args.streams)
+        cfg = dubozen_config(cfg, args.mixers, args.ffn, args.experts, args.top, args.streams, args.value_size)
         what = "dense feed-forward" if args.ffn == "dense" else f"{args.top} of {args.experts} experts"
         model_name = f"Dubozen ({args.mixers} mixers, {what}, {args.streams or 'no'} streams) at {NAMES[args.model]} sizes"
     elif args.mixers == "parallel":

@@ -64,9 +64,10 @@ CONFIGS = {
                          attention(8, 2, 32, 64, 0.18, 16, 10000.0, v_mix=True, mlp=dense(96)),
                          parallel(softmax_attention(2, 2, 32, 32, 0.18, 16, 10000.0), 4, 32, 32, [0.6, 0.8, 0.95, 0.999], 0.6, 0.5,
                                   mlp=moe(6, 1, 32, 1.0))]),
-    # keys and values of 32 and of 128 under a sink (the other two sizes the matrix cores serve), two streams
+    # keys of 32 over values of 16 (padded to 32 in the pages) and keys and values of 128 under a sink (the other two sizes the
+    # matrix cores serve), two streams
     "squares": dict(architecture="Dubozen", width=64, vocab=100, norm=dict(eps=1e-6), streams=2,
-                    layers=[attention(4, 1, 32, 32, 0.2, 32, 10000.0, v_mix=False, mlp=dense(48)),
+                    layers=[attention(4, 1, 32, 16, 0.2, 32, 10000.0, v_mix=False, mlp=dense(48)),
                             attention(2, 2, 128, 128, 0.09, 64, 10000.0, v_mix=False, mlp=None),
                             parallel(softmax_attention(4, 2, 128, 128, 0.09, 32, 10000.0), 1, 128, 128, [0.98], 0.7, 0.7, mlp=moe(4, 2, 32, 1.5, 2, 1)),
                             parallel(softmax_attention(2, 1, 32, 32, 0.2, 8, 100.0), 2, 16, 48, [0.9, 0.7], 1.0, 0.5, mlp=dense(64))]),

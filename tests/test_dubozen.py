@@ -43,6 +43,9 @@ def test_streams_are_opened_and_closed_by_layers_of_their_own():
     kv = sorted((n.kv_heads, n.head_dim, n.v_dim, c) for n, c in model.cache_groups if type(n).__name__ == "PagedKVNeed")
     # keys and values per softmax attention: (kv heads, key size, value size if it differs) and how many layers share the need
     assert kv == [(1, 8, 10, 1), (1, 16, None, 1), (2, 8, None, 1), (2, 12, 24, 1), (2, 16, 24, 1)]
+    # values smaller than keys of a size the matrix cores take are padded to the keys' size in the pages: no value size of their own
+    kv = sorted((n.kv_heads, n.head_dim, n.v_dim) for n, c in Model(spec_of(dm.CONFIGS["squares"])[1]).cache_groups if type(n).__name__ == "PagedKVNeed")
+    assert (1, 32, None) in kv and not any(v == 16 for _, _, v in kv)
     states = sorted((tuple(n.shape), c) for n, c in model.cache_groups if type(n).__name__ == "StateNeed")
     # the linear attention's memory per request: heads x (keys x values)
     assert states == [((2, 96), 1), ((3, 96), 1)]

@@ -214,6 +214,38 @@ def test_gated_attention(ops, dtype, heads, kv, dk, dv, P, rot_dims, normed, fro
         assert np.abs(f64(out).reshape(T, heads, dv)[:3] - want[:3]).max() > 10 * bound * np.abs(want[:3]).max()
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("heads,kv,dk,dv", [(4, 2, 64, 48), (2, 1, 32, 8), (3, 3, 128, 100)])
+def test_values_padded_to_the_keys_size_in_the_pages(ops, dtype, heads, kv, dk, dv):
+    """Pages with room for values of the keys' size: the rows beyond the value's size are written as zeros, and the attention
+    over them gives the bits it gives over pages without the padding."""
+    rng = np.random.default_rng(dk + dv)
+    T, P = 75, 16
+    nq, nk, nv = heads * dk, kv * dk, kv * dv
+    proj = rng.normal(size=(T, nq + nk + nv + heads * dv))
+    sink = dev(rng.normal(0.5, 1.0, size=heads))
+    table, n_pages = paged(rng, T, P)
+    pos, slots = np.arange(T, dtype=np.int32), np.zeros(T, dtype=np.int32)
+    args = (dev(pos, torch.int32), dev(slots, torch.int32), dev(table, torch.int32))
+    outs = []
+    for rows in (dv, dk):
+        pool = torch.full((n_pages, kv, P, dk + rows), float("nan"), device="cuda", dtype=DT[dtype])
+        q_out = torch.empty(T, nq, device="cuda", dtype=DT[dtype])
+        ops.gated_qkv_prep(dev(proj), None, None, None, None, *args, pool, q_out, heads, kv, dk, dv, (0, nq, nq + nk))
+        flat = f64(pool).reshape(n_pages, -1)
+        for t in (0, P - 1, P, T - 1):
+            vals = flat[table[0, t // P]][kv * P * dk:].reshape(kv, rows, P)[:, :, t % P]
+            want = f32_round(proj[t, nq + nk:nq + nk + nv]).reshape(kv, dv)
+            if dtype == "bfloat16":
+                want = bf16_round(want)
+            assert np.array_equal(vals[:, :dv], want) and not vals[:, dv:].any(), t
+        out = torch.empty(T, heads * dv, device="cuda", dtype=DT[dtype])
+        ops.gated_attention(q_out, pool, args[2], args[0], args[1], sink, dev(proj), out, heads, kv, dk, dv, 0.2, gate_col=nq + nk + nv,
+                            gate_mode=1)
+        outs.append(f64(out))
+    assert np.isfinite(outs[0]).all() and np.array_equal(outs[0], outs[1])
+
+
 def test_values_mixed_with_the_first_layers(ops):
     """Mode 1 keeps the step's values as they are projected; mode 2 caches (1 - l) v + l kept, in 32-bit."""
     rng = np.random.default_rng(11)

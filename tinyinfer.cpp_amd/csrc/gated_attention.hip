@@ -8,7 +8,9 @@
 //   attention     causal softmax over the pages with a learned number a head in the denominator (a sink: no key, no value,
 //                 not scaled) and a sigmoid gate on the output, one number an entry or one a head, read from the 32-bit sums
 //
-// A page is K [n_kv][P][dk] | V [n_kv][dv][P], as the other attention kernels of keys and values of their own sizes read it.
+// A page is K [n_kv][P][dk] | V [n_kv][dvr][P], as the other attention kernels of keys and values of their own sizes read it;
+// dvr >= dv rows a value head: rows beyond dv are written as zeros (values padded to the keys' size, so that kernels that
+// hold keys and values of one size can read the pages).
 #include "common.h"
 #include "tinyinfer_kernels.h"
 
@@ -36,7 +38,7 @@ gated_qkv_prep_kernel(const float* __restrict__ proj, int ld, int off_q, int off
                       const float* __restrict__ rope_table, int table_len, float mag, int rot_dims, int mix_mode,
                       const float* __restrict__ mix_lambda, float* __restrict__ v_kept, const int* __restrict__ pos,
                       const int* __restrict__ slot, const int* __restrict__ table, int table_stride, T* __restrict__ pool,
-                      T* __restrict__ q_out, int n_head, int n_kv, int dk, int dv, int P) {
+                      T* __restrict__ q_out, int n_head, int n_kv, int dk, int dv, int dvr, int P) {
   __shared__ float s_h[256];
   const int m = blockIdx.x, unit = blockIdx.y, lane = threadIdx.x;
   const int p = pos[m];
@@ -47,7 +49,7 @@ gated_qkv_prep_kernel(const float* __restrict__ proj, int ld, int off_q, int off
   const float* nw = is_q ? q_w : k_w;
   const int page = table[(size_t)slot[m] * table_stride + p / P];
   const int r = p % P;
-  T* base = pool + (size_t)max(page, 0) * ((size_t)n_kv * P * (dk + dv));
+  T* base = pool + (size_t)max(page, 0) * ((size_t)n_kv * P * (dk + dvr));
   float v[GA_MAX_DPL];
   float ss = 0.f;
 #pragma unroll
@@ -58,7 +60,7 @@ gated_qkv_prep_kernel(const float* __restrict__ proj, int ld, int off_q, int off
   }
   if (!is_q && off_v < 0 && page >= 0) {
     // the values are the keys as projected: before norm and rotation
-    T* vbase = base + (size_t)n_kv * P * dk + (size_t)h * dv * P + r;
+    T* vbase = base + (size_t)n_kv * P * dk + (size_t)h * dvr * P + r;
 #pragma unroll
     for (int i = 0; i < GA_MAX_DPL; ++i) {
       const int d = lane + i * TI_WAVE;
@@ -112,11 +114,14 @@ gated_qkv_prep_kernel(const float* __restrict__ proj, int ld, int off_q, int off
   const float* vs = row + off_v + (size_t)h * dv;
   float* kept = v_kept ? v_kept + ((size_t)m * n_kv + h) * dv : nullptr;
   const float lam = mix_mode == 2 ? mix_lambda[0] : 0.f;
-  T* vbase = base + (size_t)n_kv * P * dk + (size_t)h * dv * P + r;
-  for (int d = lane; d < dv; d += TI_WAVE) {
-    float x = vs[d];
-    if (mix_mode == 1) kept[d] = x;                                   // the layer whose values the later ones mix in
-    else if (mix_mode == 2) x = fmaf(lam, kept[d], (1.0f - lam) * x);
+  T* vbase = base + (size_t)n_kv * P * dk + (size_t)h * dvr * P + r;
+  for (int d = lane; d < dvr; d += TI_WAVE) {
+    float x = 0.f;                                                    // rows beyond the value's size: zeros
+    if (d < dv) {
+      x = vs[d];
+      if (mix_mode == 1) kept[d] = x;                                 // the layer whose values the later ones mix in
+      else if (mix_mode == 2) x = fmaf(lam, kept[d], (1.0f - lam) * x);
+    }
     if (page >= 0) st<T>(vbase + (size_t)d * P, x);
   }
 }
@@ -125,10 +130,11 @@ extern "C" int ti_gated_qkv_prep(int dtype, const float* proj, int ld, int off_q
                                  const float* k_w, float eps, const float* inv_freq, const float* rope_table, int table_len,
                                  float mag, int rot_dims, int mix_mode, const float* mix_lambda, float* v_kept, const int* pos,
                                  const int* slot, const int* table, int table_stride, void* pool, void* q_out, int M, int n_head,
-                                 int n_kv, int dk, int dv, int page_size, hipStream_t stream) {
-  TI_REQUIRE(n_head > 0 && n_kv > 0 && dk > 0 && dk <= 256 && dv > 0 && dv <= 256 && page_size > 0 && table_stride > 0 &&
-                 n_head + n_kv <= 65535,
-             "gated_qkv_prep: bad sizes heads=%d kv_heads=%d dk=%d dv=%d page=%d", n_head, n_kv, dk, dv, page_size);
+                                 int n_kv, int dk, int dv, int dv_rows, int page_size, hipStream_t stream) {
+  const int dvr = dv_rows > 0 ? dv_rows : dv;
+  TI_REQUIRE(n_head > 0 && n_kv > 0 && dk > 0 && dk <= 256 && dv > 0 && dv <= 256 && dvr >= dv && dvr <= 256 && page_size > 0 &&
+                 table_stride > 0 && n_head + n_kv <= 65535,
+             "gated_qkv_prep: bad sizes heads=%d kv_heads=%d dk=%d dv=%d (%d rows) page=%d", n_head, n_kv, dk, dv, dvr, page_size);
   TI_REQUIRE(!inv_freq || (rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= dk),
              "gated_qkv_prep: %d rotated entries do not fit a head of %d (even, at most the head)", rot_dims, dk);
   TI_REQUIRE(off_v >= 0 || dv == dk, "gated_qkv_prep: values that are the keys have the keys' size (%d, not %d)", dk, dv);
@@ -142,39 +148,48 @@ extern "C" int ti_gated_qkv_prep(int dtype, const float* proj, int ld, int off_q
     gated_qkv_prep_kernel<float><<<grid, TI_WAVE, 0, stream>>>(proj, ld, off_q, off_k, off_v, q_w, k_w, eps, inv_freq, rope_table,
                                                                table_len, mag, rot_dims, mix_mode, mix_lambda, v_kept, pos, slot,
                                                                table, table_stride, (float*)pool, (float*)q_out, n_head, n_kv, dk,
-                                                               dv, page_size);
+                                                               dv, dvr, page_size);
   else if (dtype == TI_BF16)
     gated_qkv_prep_kernel<bf16_t><<<grid, TI_WAVE, 0, stream>>>(proj, ld, off_q, off_k, off_v, q_w, k_w, eps, inv_freq, rope_table,
                                                                 table_len, mag, rot_dims, mix_mode, mix_lambda, v_kept, pos, slot,
                                                                 table, table_stride, (bf16_t*)pool, (bf16_t*)q_out, n_head, n_kv,
-                                                                dk, dv, page_size);
+                                                                dk, dv, dvr, page_size);
   else
     TI_REQUIRE(false, "gated_qkv_prep: unknown dtype %d", dtype);
   TI_LAUNCH_CHECK();
   return 0;
 }
 
-// The gate on its own, behind attention kernels that do not take it in: a[m, h dv + d] *= sigmoid(gate[m, h dv + d] or gate[m, h])
+// The gate on its own, behind attention kernels that do not take it in: out[m, h dv + d] = src[m, h src_dv + d] times
+// sigmoid(gate[m, h dv + d] or gate[m, h]) (gate null: times one).  src_dv > dv: the heads of src are padded and come out packed;
+// src may be out where src_dv = dv.
 template <typename T>
-__global__ void sigmoid_gate_kernel(T* __restrict__ a, const float* __restrict__ gate, int gate_ld, int gate_mode, long n, int W, int dv) {
+__global__ void sigmoid_gate_kernel(const T* __restrict__ src, int src_dv, T* __restrict__ out, const float* __restrict__ gate,
+                                    int gate_ld, int gate_mode, long n, int n_head, int dv) {
+  const int W = n_head * dv;
   for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
     const long m = i / W;
-    const int c = (int)(i % W);
-    const float z = gate[m * gate_ld + (gate_mode == 1 ? c : c / dv)];
-    st<T>(a + i, ld<T>(a + i) * (1.0f / (1.0f + expf(-z))));
+    const int c = (int)(i % W), h = c / dv;
+    float y = ld<T>(src + m * ((long)n_head * src_dv) + (long)h * src_dv + (c - h * dv));
+    if (gate) y *= 1.0f / (1.0f + expf(-gate[m * gate_ld + (gate_mode == 1 ? c : h)]));
+    st<T>(out + i, y);
   }
 }
 
-extern "C" int ti_sigmoid_gate(int dtype, void* a, const float* gate, int gate_ld, int gate_mode, int M, int n_head, int dv,
-                               hipStream_t stream) {
-  TI_REQUIRE(M >= 0 && n_head > 0 && dv > 0 && gate && ((gate_mode == 1 && gate_ld >= n_head * dv) || (gate_mode == 2 && gate_ld >= n_head)),
-             "sigmoid_gate: bad sizes M=%d heads=%d dv=%d gate mode %d in rows of %d", M, n_head, dv, gate_mode, gate_ld);
+extern "C" int ti_sigmoid_gate(int dtype, const void* src, int src_dv, void* out, const float* gate, int gate_ld, int gate_mode, int M,
+                               int n_head, int dv, hipStream_t stream) {
+  TI_REQUIRE(M >= 0 && n_head > 0 && dv > 0 && src_dv >= dv && (src != out || src_dv == dv) &&
+                 (!gate || (gate_mode == 1 && gate_ld >= n_head * dv) || (gate_mode == 2 && gate_ld >= n_head)),
+             "sigmoid_gate: bad sizes M=%d heads=%d dv=%d (from %d) gate mode %d in rows of %d", M, n_head, dv, src_dv, gate_mode, gate_ld);
   if (M == 0) return 0;
   const long n = (long)M * n_head * dv;
   const unsigned blocks = (unsigned)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
-  if (dtype == TI_F32) sigmoid_gate_kernel<float><<<blocks, 256, 0, stream>>>((float*)a, gate, gate_ld, gate_mode, n, n_head * dv, dv);
-  else if (dtype == TI_BF16) sigmoid_gate_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)a, gate, gate_ld, gate_mode, n, n_head * dv, dv);
-  else TI_REQUIRE(false, "sigmoid_gate: unknown dtype %d", dtype);
+  if (dtype == TI_F32)
+    sigmoid_gate_kernel<float><<<blocks, 256, 0, stream>>>((const float*)src, src_dv, (float*)out, gate, gate_ld, gate_mode, n, n_head, dv);
+  else if (dtype == TI_BF16)
+    sigmoid_gate_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)src, src_dv, (bf16_t*)out, gate, gate_ld, gate_mode, n, n_head, dv);
+  else
+    TI_REQUIRE(false, "sigmoid_gate: unknown dtype %d", dtype);
   TI_LAUNCH_CHECK();
   return 0;
 }
@@ -192,7 +207,7 @@ __global__ void __launch_bounds__(256)
 gated_attention_kernel(const T* __restrict__ q, const T* __restrict__ pool, const int* __restrict__ table, int table_stride,
                        const int* __restrict__ pos, const int* __restrict__ slot, const float* __restrict__ sink,
                        const float* __restrict__ gate, int gate_ld, int gate_mode, T* __restrict__ out, int n_head, int n_kv,
-                       int dk, int dv, int P, float scale, int window) {
+                       int dk, int dv, int dvr, int P, float scale, int window) {
   constexpr int HD = DPL * GA_LANES;
   __shared__ float s_o[GA_GROUPS][HD];
   __shared__ float s_m[GA_GROUPS], s_l[GA_GROUPS];
@@ -202,9 +217,9 @@ gated_attention_kernel(const T* __restrict__ q, const T* __restrict__ pool, cons
   const int p_q = pos[m];
   const int lo = (window > 0 && p_q - window + 1 > 0) ? p_q - window + 1 : 0;
   const int* tab = table + (size_t)slot[m] * table_stride;
-  const size_t page_elems = (size_t)n_kv * P * (dk + dv);
+  const size_t page_elems = (size_t)n_kv * P * (dk + dvr);
   const size_t k_off = (size_t)kvh * P * dk;
-  const size_t v_off = (size_t)n_kv * P * dk + (size_t)kvh * dv * P;
+  const size_t v_off = (size_t)n_kv * P * dk + (size_t)kvh * dvr * P;
 
   float qv[DPL], o[DPL];
   const T* qh = q + ((size_t)m * n_head + h) * dk;
@@ -271,11 +286,11 @@ gated_attention_kernel(const T* __restrict__ q, const T* __restrict__ pool, cons
 template <typename T>
 static int launch_gated(int dpl, dim3 grid, const void* q, const void* pool, const int* table, int table_stride, const int* pos,
                         const int* slot, const float* sink, const float* gate, int gate_ld, int gate_mode, void* out, int n_head,
-                        int n_kv, int dk, int dv, int P, float scale, int window, hipStream_t stream) {
+                        int n_kv, int dk, int dv, int dvr, int P, float scale, int window, hipStream_t stream) {
 #define GA_CASE(D)                                                                                                       \
   case D:                                                                                                                \
     gated_attention_kernel<T, D><<<grid, 256, 0, stream>>>((const T*)q, (const T*)pool, table, table_stride, pos, slot, sink, \
-                                                           gate, gate_ld, gate_mode, (T*)out, n_head, n_kv, dk, dv, P, scale, \
+                                                           gate, gate_ld, gate_mode, (T*)out, n_head, n_kv, dk, dv, dvr, P, scale, \
                                                            window);                                                      \
     break;
   switch (dpl) {
@@ -291,8 +306,10 @@ static int launch_gated(int dpl, dim3 grid, const void* q, const void* pool, con
 // q: [M, n_head, dk], out: [M, n_head, dv] in T
 extern "C" int ti_gated_attention_rows(int dtype, const void* q, const void* pool, const int* table, int table_stride,
                                        const int* pos, const int* slot, const float* sink, const float* gate, int gate_ld,
-                                       int gate_mode, void* out, int M, int n_head, int n_kv, int dk, int dv, int page_size,
+                                       int gate_mode, void* out, int M, int n_head, int n_kv, int dk, int dv, int dv_rows, int page_size,
                                        float scale, int window, hipStream_t stream) {
+  const int dvr = dv_rows > 0 ? dv_rows : dv;
+  TI_REQUIRE(dvr >= dv && dvr <= 256, "gated attention: %d rows a value head do not hold values of %d", dvr, dv);
   TI_REQUIRE(dk >= 1 && dk <= 256 && dv >= 1 && dv <= 256, "gated attention: key size %d / value size %d are not served (up to 256)",
              dk, dv);
   TI_REQUIRE(n_head > 0 && n_kv > 0 && n_head % n_kv == 0 && n_head <= 65535, "gated attention: heads %d / kv_heads %d", n_head, n_kv);
@@ -306,10 +323,10 @@ extern "C" int ti_gated_attention_rows(int dtype, const void* q, const void* poo
   int rc;
   if (dtype == TI_F32)
     rc = launch_gated<float>(dpl, grid, q, pool, table, table_stride, pos, slot, sink, gate, gate_ld, gate_mode, out, n_head, n_kv, dk,
-                             dv, page_size, scale, window, stream);
+                             dv, dvr, page_size, scale, window, stream);
   else if (dtype == TI_BF16)
     rc = launch_gated<bf16_t>(dpl, grid, q, pool, table, table_stride, pos, slot, sink, gate, gate_ld, gate_mode, out, n_head, n_kv,
-                              dk, dv, page_size, scale, window, stream);
+                              dk, dv, dvr, page_size, scale, window, stream);
   else
     TI_REQUIRE(false, "gated attention: unknown dtype %d", dtype);
   TI_REQUIRE(rc == 0, "gated attention: no kernel for sizes %d / %d", dk, dv);

@@ -216,19 +216,23 @@ int ti_hyper_write_read(int out_dtype, float* streams, long stream_stride, int S
 // proj f32 [M, ld] holds q (n_head x dk), k (n_kv x dk) and v (n_kv x dv; off_v < 0: the values are the keys as projected) from
 // the given columns on.  q_w / k_w (null: none): RMS norm of every head before the rotation of its first rot_dims entries.
 // mix_mode 1: the values also go to v_kept f32 [M, n_kv dv]; 2: v <- (1 - lambda) v + lambda v_kept (lambda: one float in
-// device memory).  q to q_out, k and v into the pages K [n_kv][P][dk] | V [n_kv][dv][P]
+// device memory).  q to q_out, k and v into the pages K [n_kv][P][dk] | V [n_kv][dv_rows][P] (dv_rows >= dv, 0: dv; rows of a
+// value head beyond dv are written as zeros: values padded to the keys' size for kernels that hold both at one size)
 int ti_gated_qkv_prep(int dtype, const float* proj, int ld, int off_q, int off_k, int off_v, const float* q_w, const float* k_w,
                       float eps, const float* inv_freq, const float* rope_table, int table_len, float mag, int rot_dims,
                       int mix_mode, const float* mix_lambda, float* v_kept, const int* pos, const int* slot, const int* table,
-                      int table_stride, void* pool, void* q_out, int M, int n_head, int n_kv, int dk, int dv, int page_size,
-                      hipStream_t stream);
-// a (T [M, n_head dv]) *= sigmoid(gate), gate f32 rows of gate_ld floats: entry h dv + d (gate_mode 1) or h (gate_mode 2)
-int ti_sigmoid_gate(int dtype, void* a, const float* gate, int gate_ld, int gate_mode, int M, int n_head, int dv, hipStream_t stream);
+                      int table_stride, void* pool, void* q_out, int M, int n_head, int n_kv, int dk, int dv, int dv_rows,
+                      int page_size, hipStream_t stream);
+// out (T [M, n_head dv]) = src (T [M, n_head src_dv], the first dv of every head) times sigmoid(gate), gate f32 rows of gate_ld
+// floats: entry h dv + d (gate_mode 1) or h (gate_mode 2); gate null: times one; src may be out where src_dv = dv
+int ti_sigmoid_gate(int dtype, const void* src, int src_dv, void* out, const float* gate, int gate_ld, int gate_mode, int M,
+                    int n_head, int dv, hipStream_t stream);
 // causal softmax attention of every row over such pages; sink f32 [n_head] (null: none) joins the denominator; gate (null:
 // none) f32 rows of gate_ld floats, the output times sigmoid of entry h dv + d (gate_mode 1) or h (gate_mode 2)
 int ti_gated_attention_rows(int dtype, const void* q, const void* pool, const int* table, int table_stride, const int* pos,
                             const int* slot, const float* sink, const float* gate, int gate_ld, int gate_mode, void* out, int M,
-                            int n_head, int n_kv, int dk, int dv, int page_size, float scale, int window, hipStream_t stream);
+                            int n_head, int n_kv, int dk, int dv, int dv_rows, int page_size, float scale, int window,
+                            hipStream_t stream);
 
 // ---- libti_linear_attention: linear attention with a fixed decay per head, and the gated norm behind it
 // S_t = decay_h S_(t-1) + k_t v_t^T, o_t = S_t^T q_t with q, k, v = silu of the given columns of proj f32 [M, ld]; state f32

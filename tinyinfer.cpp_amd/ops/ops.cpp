@@ -1263,6 +1263,15 @@ void Ops::hyper_write(const Tensor& streams, const Tensor& mix, const Tensor& ba
   check("hyper", rc, "hyper_write");
 }
 
+// the rows a value head has in the pages of `pool`: dv, or more where the values are padded (to the keys' size)
+static int value_rows(const char* what, const Tensor& pool, int kv_heads, int dk, int dv) {
+  require(pool.ndim == 4 && kv_heads > 0 && (pool.shape[1] * pool.shape[3]) % kv_heads == 0,
+          std::string(what) + ": pool " + pool.describe() + " does not hold " + std::to_string(kv_heads) + " kv heads");
+  const int64_t rows = pool.shape[1] * pool.shape[3] / kv_heads - dk;
+  require(rows >= dv && rows <= 256, std::string(what) + ": pool " + pool.describe() + " has no room for values of " + std::to_string(dv));
+  return (int)rows;
+}
+
 void Ops::gated_qkv_prep(const Tensor& proj, const QkvColumns& cols, const Tensor& q_w, const Tensor& k_w, float eps, const Rotation& rot,
                          const ValueMix& mix, const int* positions, const int* slots, const CacheView& view, const Tensor& pool,
                          const Tensor& q_out, int heads, int kv_heads, int dk, int dv) {
@@ -1277,14 +1286,15 @@ void Ops::gated_qkv_prep(const Tensor& proj, const QkvColumns& cols, const Tenso
   require(mix.mode == 0 || (mix.kept.dtype == DType::F32 && mix.kept.contiguous() && mix.kept.numel() == M * kv_heads * dv &&
                             (mix.mode == 1 || (mix.lambda.dtype == DType::F32 && mix.lambda.numel() == 1))),
           "gated_qkv_prep: the kept values " + mix.kept.describe() + " or the factor do not fit");
-  check_split_pool("gated_qkv_prep", pool, kv_heads, dk, dv, q_out.dtype);
+  const int dvr = value_rows("gated_qkv_prep", pool, kv_heads, dk, dv);
+  check_split_pool("gated_qkv_prep", pool, kv_heads, dk, dvr, q_out.dtype);
   const int rot_dims = rot.inv_freq ? (rot.dims > 0 ? rot.dims : dk) : 0;
   int rc = KERNEL("gated_attention", ti_gated_qkv_prep)(
       code(q_out.dtype, "gated_qkv_prep"), (const float*)proj.data, (int)proj.shape[1], cols.q, cols.k, cols.v,
       q_w.defined() ? (const float*)q_w.data : nullptr, k_w.defined() ? (const float*)k_w.data : nullptr, eps, rot.inv_freq, rot.table,
       rot.table_len, rot.mag, rot_dims, mix.mode, mix.mode == 2 ? (const float*)mix.lambda.data : nullptr,
       mix.mode ? (float*)mix.kept.data : nullptr, positions, slots, view.table, view.table_width, pool.data, q_out.data, (int)M, heads,
-      kv_heads, dk, dv, (int)pool.shape[2], (hipStream_t)launch_stream());
+      kv_heads, dk, dv, dvr, (int)pool.shape[2], (hipStream_t)launch_stream());
   check("gated_attention", rc, "gated_qkv_prep");
 }
 
@@ -1303,15 +1313,19 @@ void Ops::gated_attention(const Tensor& q, const Tensor& pool, const CacheView& 
                 gate.proj.shape[0] == M && gate.col >= 0 && gate.col + need <= gate.proj.shape[1],
             "gated_attention: the gate's columns do not lie inside proj " + gate.proj.describe());
   }
-  check_split_pool("gated_attention", pool, kv_heads, dk, dv, q.dtype);
+  const int dvr = value_rows("gated_attention", pool, kv_heads, dk, dv);
+  check_split_pool("gated_attention", pool, kv_heads, dk, dvr, q.dtype);
   const float* gate_ptr = gate.mode ? (const float*)gate.proj.data + gate.col : nullptr;
-  if (work && ws && dk == dv && q.dtype == DType::BF16 && use.fast_attention && kernel_library_available("attention_bf16") &&
+  if (work && ws && dk == dvr && q.dtype == DType::BF16 && use.fast_attention && kernel_library_available("attention_bf16") &&
       (dk == 32 || dk == 64 || dk == 128) && pool.shape[2] % 16 == 0) {
-    // the matrix-core kernels of plain attention, the sink joining where they finish a column; the gate behind them
-    attention(*work, *ws, view, q, pool, out, heads, kv_heads, dk, scale, window, 0.f, sink.defined() ? (const float*)sink.data : nullptr);
-    if (gate.mode) {
-      int rc = KERNEL("gated_attention", ti_sigmoid_gate)(code(out.dtype, "gated_attention"), out.data, gate_ptr, (int)gate.proj.shape[1],
-                                                          gate.mode, (int)M, heads, dv, (hipStream_t)launch_stream());
+    // the matrix-core kernels of plain attention (values of the keys' size, padded with zeros in the pages where they are
+    // smaller), the sink joining where they finish a column; the gate behind them, which also packs padded heads
+    Tensor wide = dv == dk ? out : ws->tensor("attn.out_padded", out.dtype, {M, (int64_t)heads * dk});
+    attention(*work, *ws, view, q, pool, wide, heads, kv_heads, dk, scale, window, 0.f, sink.defined() ? (const float*)sink.data : nullptr);
+    if (gate.mode || dv != dk) {
+      int rc = KERNEL("gated_attention", ti_sigmoid_gate)(code(out.dtype, "gated_attention"), wide.data, dk, out.data, gate_ptr,
+                                                          gate.mode ? (int)gate.proj.shape[1] : 0, gate.mode, (int)M, heads, dv,
+                                                          (hipStream_t)launch_stream());
       check("gated_attention", rc, "gated_attention(gate)");
     }
     took("[mfma]");
@@ -1321,8 +1335,8 @@ void Ops::gated_attention(const Tensor& q, const Tensor& pool, const CacheView& 
   int rc = KERNEL("gated_attention", ti_gated_attention_rows)(
       code(q.dtype, "gated_attention"), q.data, pool.data, view.table, view.table_width, positions, slots,
       sink.defined() ? (const float*)sink.data : nullptr, gate.mode ? (const float*)gate.proj.data + gate.col : nullptr,
-      gate.mode ? (int)gate.proj.shape[1] : 0, gate.mode, out.data, (int)M, heads, kv_heads, dk, dv, (int)pool.shape[2], scale, window,
-      (hipStream_t)launch_stream());
+      gate.mode ? (int)gate.proj.shape[1] : 0, gate.mode, out.data, (int)M, heads, kv_heads, dk, dv, dvr, (int)pool.shape[2], scale,
+      window, (hipStream_t)launch_stream());
   check("gated_attention", rc, "gated_attention");
 }
 

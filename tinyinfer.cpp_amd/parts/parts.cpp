@@ -716,7 +716,10 @@ class Attention final : public MixerPart {
     n.kind = CacheNeed::PagedKV;
     n.kv_heads = kv_heads;
     n.head_dim = head_dim;
-    n.v_dim = v_dim != head_dim ? v_dim : 0;
+    // gated layers whose values are smaller than keys of a size the matrix cores take: the pages hold the values padded with
+    // zeros to the keys' size, so that the kernels that hold keys and values of one size read them
+    const bool padded = gated && v_dim < head_dim && (head_dim == 32 || head_dim == 64 || head_dim == 128);
+    n.v_dim = (v_dim != head_dim && !padded) ? v_dim : 0;
     n.window = window;
     return n;
   }
